@@ -1,0 +1,205 @@
+"""ctypes binding of libodc_hip.so (the C ABI declared in include/odc_hip.h).
+
+This is the only place where Python touches the native library. It plays the part that
+``odc/primitives/__init__.py:16-29`` plays in the reference (import the native extension, fail
+hard when it has not been built): there is no Python or CPU fallback behind any entry point.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+import threading
+from pathlib import Path
+
+_PKG_DIR = Path(__file__).resolve().parent
+CSRC_DIR = _PKG_DIR / "csrc"
+INCLUDE_DIR = _PKG_DIR.parent / "include"
+LIB_PATH = CSRC_DIR / "libodc_hip.so"
+SOURCES = [CSRC_DIR / "odc_hip.hip"]
+
+# every symbol include/odc_hip.h declares
+EXPORTED_SYMBOLS = (
+    "odc_arena_create",
+    "odc_arena_destroy",
+    "odc_arena_alloc",
+    "odc_arena_free",
+    "odc_arena_reset",
+    "odc_arena_get_info",
+    "odc_arena_ptr",
+    "odc_arena_locate",
+    "odc_gather",
+    "odc_scatter_accumulate",
+    "odc_clear",
+    "odc_last_error",
+    "odc_abi_version",
+    "odc_set_option",
+    "odc_get_option",
+)
+
+ABI_VERSION = 1
+MAX_ITEMS_PER_LAUNCH = 32
+
+ODC_OK = 0
+ODC_ERR_INVALID = -1
+ODC_ERR_NOMEM = -2
+ODC_ERR_HIP = -3
+ODC_ERR_UNSUPPORTED = -4
+ODC_ERR_NOT_FOUND = -5
+ODC_ERR_NO_BACKING = -6
+
+ODC_ARENA_DEVICE = 0
+ODC_ARENA_NO_BACKING = 1
+
+DTYPE_BF16 = 0
+DTYPE_F16 = 1
+DTYPE_F32 = 2
+
+
+class OdcNativeError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libodc_hip: {message} (status {code})")
+        self.code = code
+        self.message = message
+
+
+class ArenaInfo(ctypes.Structure):
+    _fields_ = [
+        ("world_size", ctypes.c_uint32),
+        ("device", ctypes.c_int32),
+        ("flags", ctypes.c_uint32),
+        ("n_allocations", ctypes.c_uint32),
+        ("bytes_per_rank", ctypes.c_uint64),
+        ("rank_stride", ctypes.c_uint64),
+        ("base", ctypes.c_uint64),
+        ("bytes_in_use", ctypes.c_uint64),
+        ("high_water", ctypes.c_uint64),
+    ]
+
+
+class GatherItem(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("src_offset", ctypes.c_uint64),
+        ("shard_bytes", ctypes.c_uint64),
+    ]
+
+
+class AccumItem(ctypes.Structure):
+    _fields_ = [
+        ("grad", ctypes.c_void_p),
+        ("grad_elems", ctypes.c_uint64),
+        ("acc_offset", ctypes.c_uint64),
+        ("shard_elems", ctypes.c_uint64),
+    ]
+
+
+class Span(ctypes.Structure):
+    _fields_ = [("offset", ctypes.c_uint64), ("nbytes", ctypes.c_uint64)]
+
+
+def hipcc_command(output: Path = LIB_PATH) -> list[str]:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    return [
+        hipcc,
+        "-O3",
+        "-std=c++17",
+        "--offload-arch=gfx950",
+        # keep hipcc from fusing float pairs into packed-fp32 instructions
+        "-Xclang",
+        "-target-feature",
+        "-Xclang",
+        "-packed-fp32-ops",
+        "-fPIC",
+        "-shared",
+        f"-I{INCLUDE_DIR}",
+        "-o",
+        str(output),
+        *[str(s) for s in SOURCES],
+    ]
+
+
+def build_library(verbose: bool = False) -> Path:
+    """Compile libodc_hip.so in-tree for gfx950 (works without a GPU)."""
+    cmd = hipcc_command()
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or proc.returncode != 0:
+        print(" ".join(cmd))
+        print(proc.stdout)
+        print(proc.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}")
+    return LIB_PATH
+
+
+_lib = None
+_lib_lock = threading.Lock()
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    vp, u32, u64, i64, ci = (
+        ctypes.c_void_p,
+        ctypes.c_uint32,
+        ctypes.c_uint64,
+        ctypes.c_int64,
+        ctypes.c_int,
+    )
+    P = ctypes.POINTER
+    lib.odc_arena_create.argtypes = [u32, u64, u32, P(vp)]
+    lib.odc_arena_destroy.argtypes = [vp]
+    lib.odc_arena_alloc.argtypes = [vp, u64, P(u64)]
+    lib.odc_arena_free.argtypes = [vp, u64]
+    lib.odc_arena_reset.argtypes = [vp]
+    lib.odc_arena_get_info.argtypes = [vp, P(ArenaInfo)]
+    lib.odc_arena_ptr.argtypes = [vp, u32, u64]
+    lib.odc_arena_ptr.restype = vp
+    lib.odc_arena_locate.argtypes = [vp, vp, P(u32), P(u64), P(u64)]
+    lib.odc_gather.argtypes = [vp, P(GatherItem), u32, u32, vp]
+    lib.odc_scatter_accumulate.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
+    lib.odc_clear.argtypes = [vp, P(Span), u32, vp]
+    lib.odc_last_error.argtypes = []
+    lib.odc_last_error.restype = ctypes.c_char_p
+    lib.odc_abi_version.argtypes = []
+    lib.odc_set_option.argtypes = [ctypes.c_char_p, i64]
+    lib.odc_get_option.argtypes = [ctypes.c_char_p, P(i64)]
+    for name in EXPORTED_SYMBOLS:
+        fn = getattr(lib, name)
+        if name not in ("odc_arena_ptr", "odc_last_error"):
+            fn.restype = ci
+
+
+def load() -> ctypes.CDLL:
+    """Load the in-tree library; raise if it is missing or has the wrong ABI."""
+    global _lib
+    with _lib_lock:
+        if _lib is None:
+            if not LIB_PATH.exists():
+                raise ImportError(
+                    f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; "
+                    "g.build()'` (needs hipcc). There is no fallback path."
+                )
+            lib = ctypes.CDLL(str(LIB_PATH))
+            _declare(lib)
+            got = lib.odc_abi_version()
+            if got != ABI_VERSION:
+                raise ImportError(f"{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}: rebuild it")
+            _lib = lib
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != ODC_OK:
+        raise OdcNativeError(status, load().odc_last_error().decode("utf-8", "replace"))
+
+
+def set_option(name: str, value: int) -> None:
+    check(load().odc_set_option(name.encode(), int(value)))
+
+
+def get_option(name: str) -> int:
+    out = ctypes.c_int64(0)
+    check(load().odc_get_option(name.encode(), ctypes.byref(out)))
+    return out.value

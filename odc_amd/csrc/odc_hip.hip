@@ -1,0 +1,846 @@
+// libodc_hip.so — gfx950 (MI355X, CDNA4) implementation of the C ABI in include/odc_hip.h.
+//
+// Three streaming kernels, all HBM-bandwidth bound (no MFMA, no LDS):
+//   gather_kernel  : W shard regions -> one flat buffer            (read 1 B + write 1 B per byte)
+//   accum_kernel   : acc_r += widen(grad chunk r), in place        (bf16->fp32: 10 B per element)
+//   clear_kernel   : zero a span in every rank region              (write 1 B per byte)
+// plus the host-side symmetric arena (one hipMalloc, W rank regions, one offset valid in all).
+//
+// Launch model shared by the three kernels: the work of one launch is cut into tiles of
+// kThreads * kUnroll 16-byte vectors; 256-thread workgroups walk the tiles with a grid-stride
+// loop so that, at any instant, the whole chip streams one compact window of memory. Per-item
+// descriptors (<= ODC_MAX_ITEMS_PER_LAUNCH) travel BY VALUE in the kernel argument segment and
+// are read with scalar loads, so a call needs no device-side work list, no host->device copy and
+// no allocation; longer item lists are split over several launches.
+//
+// Each wavefront issues kUnroll independent 128-bit nontemporal loads per stream before the
+// first store: on this part the nontemporal hint on both loads and stores is worth ~15 % over
+// plain accesses for these single-touch streams.
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <string>
+
+#include "odc_hip.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// errors
+// ------------------------------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define ODC_HIP_TRY(expr)                                                                   \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      return fail(ODC_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),       \
+                  __FILE__, __LINE__);                                                      \
+  } while (0)
+
+// ------------------------------------------------------------------------------------------------
+// options
+// ------------------------------------------------------------------------------------------------
+struct Options {
+  int64_t gather_blocks_per_cu = 8;
+  int64_t accum_blocks_per_cu = 8;
+  int64_t clear_blocks_per_cu = 8;
+  int64_t rank_major = 1;
+  int64_t rank_stagger_bytes = 0;
+};
+Options g_opt;
+std::mutex g_opt_mu;
+
+int64_t* option_slot(const char* name) {
+  if (!name) return nullptr;
+  if (!strcmp(name, "gather_blocks_per_cu")) return &g_opt.gather_blocks_per_cu;
+  if (!strcmp(name, "accum_blocks_per_cu")) return &g_opt.accum_blocks_per_cu;
+  if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
+  if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
+  if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
+  return nullptr;
+}
+
+// ------------------------------------------------------------------------------------------------
+// device side
+// ------------------------------------------------------------------------------------------------
+constexpr int kThreads = 256;  // 4 wavefronts of 64 lanes
+constexpr int kUnroll = 4;     // independent 16 B accesses per lane per stream before the stores
+constexpr int kMaxItems = ODC_MAX_ITEMS_PER_LAUNCH;
+constexpr uint32_t kTileVecs = kThreads * kUnroll;      // 16 B vectors per tile
+constexpr uint32_t kTileBytes = kTileVecs * 16;         // gather / clear: 16 KiB of destination
+constexpr uint32_t kTileElems = kTileVecs * 4;          // accumulate: 4096 elements
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Per-launch descriptors, passed by value (kernel argument segment, scalar loads).
+struct GatherLaunch {
+  const uint8_t* base;   // arena base (rank 0 region)
+  uint64_t rank_stride;
+  uint32_t world;
+  uint32_t first_rank;
+  uint32_t n_items;
+  uint32_t n_tiles;
+  uint32_t rank_major;
+  uint32_t tile_prefix[kMaxItems + 1];
+  uint32_t tiles_per_seg[kMaxItems];
+  uint8_t* dst[kMaxItems];
+  uint64_t src_off[kMaxItems];
+  uint64_t seg_bytes[kMaxItems];
+};
+
+struct AccumLaunch {
+  uint8_t* base;
+  uint64_t rank_stride;
+  uint32_t world;
+  uint32_t n_items;
+  uint32_t n_tiles;
+  uint32_t rank_major;
+  uint32_t tile_prefix[kMaxItems + 1];
+  uint32_t tiles_per_seg[kMaxItems];
+  const uint8_t* grad[kMaxItems];
+  uint64_t grad_elems[kMaxItems];
+  uint64_t acc_off[kMaxItems];
+  uint64_t seg_elems[kMaxItems];
+};
+
+struct ClearLaunch {
+  uint8_t* base;
+  uint64_t rank_stride;
+  uint32_t world;
+  uint32_t n_items;
+  uint32_t n_tiles;
+  uint32_t rank_major;
+  uint32_t tile_prefix[kMaxItems + 1];
+  uint32_t tiles_per_seg[kMaxItems];
+  uint64_t off[kMaxItems];
+  uint64_t seg_bytes[kMaxItems];
+};
+
+// Tile t of a launch -> (item, rank, chunk-in-segment). Everything here is wave-uniform.
+struct TileCoord {
+  uint32_t item, rank, chunk;
+};
+
+template <class L>
+__device__ __forceinline__ TileCoord locate_tile(const L& launch, uint32_t t, uint32_t first_rank) {
+  uint32_t lo = 0, hi = launch.n_items;  // largest i with tile_prefix[i] <= t
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (launch.tile_prefix[mid] <= t) lo = mid; else hi = mid;
+  }
+  const uint32_t lt = t - launch.tile_prefix[lo];
+  const uint32_t tps = launch.tiles_per_seg[lo];
+  TileCoord c;
+  c.item = lo;
+  if (launch.rank_major) {
+    c.rank = lt / tps;
+    c.chunk = lt - c.rank * tps;
+  } else {
+    c.chunk = lt / launch.world;
+    c.rank = lt - c.chunk * launch.world;
+  }
+  c.rank += first_rank;
+  if (c.rank >= launch.world) c.rank -= launch.world;
+  return c;
+}
+
+__device__ __forceinline__ u32x4 load16_unaligned(const uint8_t* p) {
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+
+// ---- gather -------------------------------------------------------------------------------
+// Copies n bytes d[0:n] = s[0:n] with the 256 threads of the block; any alignment. Stores are
+// 16 B aligned on the destination; the source side takes whatever misalignment is left.
+__device__ __forceinline__ void copy_any(uint8_t* d, const uint8_t* s, uint32_t n) {
+  const uint32_t tid = threadIdx.x;
+  uint32_t head = (16u - (uint32_t)((uintptr_t)d & 15u)) & 15u;
+  if (head > n) head = n;
+  if (tid < head) d[tid] = s[tid];
+  d += head;
+  s += head;
+  n -= head;
+  const uint32_t nvec = n >> 4;
+  for (uint32_t v = tid; v < nvec; v += kThreads) {
+    const u32x4 x = load16_unaligned(s + (size_t)v * 16);
+    __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(d) + v);
+  }
+  const uint32_t tail = n & 15u;
+  if (tid < tail) d[(size_t)nvec * 16 + tid] = s[(size_t)nvec * 16 + tid];
+}
+
+__global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
+  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch, t, launch.first_rank);
+    const uint64_t seg = launch.seg_bytes[c.item];
+    const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride +
+                       launch.src_off[c.item] + in_seg;
+    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg + in_seg;
+    const uint64_t left = seg - in_seg;
+    if (left >= kTileBytes && ((((uintptr_t)d) | ((uintptr_t)s)) & 15u) == 0) {
+      const u32x4* sv = reinterpret_cast<const u32x4*>(s) + threadIdx.x;
+      u32x4* dv = reinterpret_cast<u32x4*>(d) + threadIdx.x;
+      u32x4 v[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(sv + u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], dv + u * kThreads);
+    } else {
+      copy_any(d, s, left < kTileBytes ? (uint32_t)left : kTileBytes);
+    }
+  }
+}
+
+// ---- clear --------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launch) {
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch, t, 0);
+    const uint64_t seg = launch.seg_bytes[c.item];
+    const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
+    uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.off[c.item] + in_seg;
+    const uint64_t left = seg - in_seg;
+    if (left >= kTileBytes && (((uintptr_t)d) & 15u) == 0) {
+      u32x4* dv = reinterpret_cast<u32x4*>(d) + threadIdx.x;
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(zero, dv + u * kThreads);
+    } else {
+      uint32_t n = left < kTileBytes ? (uint32_t)left : kTileBytes;
+      const uint32_t tid = threadIdx.x;
+      uint32_t head = (16u - (uint32_t)((uintptr_t)d & 15u)) & 15u;
+      if (head > n) head = n;
+      if (tid < head) d[tid] = 0;
+      d += head;
+      n -= head;
+      const uint32_t nvec = n >> 4;
+      for (uint32_t v = tid; v < nvec; v += kThreads)
+        __builtin_nontemporal_store(zero, reinterpret_cast<u32x4*>(d) + v);
+      const uint32_t tail = n & 15u;
+      if (tid < tail) d[(size_t)nvec * 16 + tid] = 0;
+    }
+  }
+}
+
+// ---- scatter-accumulate -------------------------------------------------------------------
+// Element codecs. Widening to fp32 is exact for all three types; narrowing rounds to nearest
+// even. The add itself is one v_add_f32 per element: no contraction, no reassociation.
+struct bf16_tag {};
+struct f16_tag {};
+struct f32_tag {};
+
+template <class T> struct Codec;
+template <> struct Codec<f32_tag> {
+  static constexpr int kBytes = 4;
+  typedef uint32_t raw_t;
+  static __device__ __forceinline__ float widen(uint32_t r) { return __uint_as_float(r); }
+  static __device__ __forceinline__ uint32_t narrow(float f) { return __float_as_uint(f); }
+};
+template <> struct Codec<bf16_tag> {
+  static constexpr int kBytes = 2;
+  typedef uint16_t raw_t;
+  static __device__ __forceinline__ float widen(uint16_t r) { return __uint_as_float((uint32_t)r << 16); }
+  static __device__ __forceinline__ uint16_t narrow(float f) {
+    const uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  }
+};
+template <> struct Codec<f16_tag> {
+  static constexpr int kBytes = 2;
+  typedef uint16_t raw_t;
+  static __device__ __forceinline__ float widen(uint16_t r) {
+    return (float)__builtin_bit_cast(_Float16, r);
+  }
+  static __device__ __forceinline__ uint16_t narrow(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+  }
+};
+
+// Four consecutive elements as raw dwords: 2 dwords for the 16-bit types, 4 for fp32.
+template <class T> struct Quad;
+template <> struct Quad<f32_tag> {
+  typedef u32x4 vec_t;
+  static __device__ __forceinline__ void widen(vec_t r, float (&f)[4]) {
+    f[0] = __uint_as_float(r.x); f[1] = __uint_as_float(r.y);
+    f[2] = __uint_as_float(r.z); f[3] = __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ vec_t narrow(const float (&f)[4]) {
+    vec_t r = {__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    return r;
+  }
+};
+template <> struct Quad<bf16_tag> {
+  typedef u32x2 vec_t;
+  static __device__ __forceinline__ void widen(vec_t r, float (&f)[4]) {
+    f[0] = __uint_as_float(r.x << 16); f[1] = __uint_as_float(r.x & 0xffff0000u);
+    f[2] = __uint_as_float(r.y << 16); f[3] = __uint_as_float(r.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ vec_t narrow(const float (&f)[4]) {
+    vec_t r;
+    r.x = (uint32_t)Codec<bf16_tag>::narrow(f[0]) | ((uint32_t)Codec<bf16_tag>::narrow(f[1]) << 16);
+    r.y = (uint32_t)Codec<bf16_tag>::narrow(f[2]) | ((uint32_t)Codec<bf16_tag>::narrow(f[3]) << 16);
+    return r;
+  }
+};
+template <> struct Quad<f16_tag> {
+  typedef u32x2 vec_t;
+  static __device__ __forceinline__ void widen(vec_t r, float (&f)[4]) {
+    f[0] = Codec<f16_tag>::widen((uint16_t)(r.x & 0xffffu)); f[1] = Codec<f16_tag>::widen((uint16_t)(r.x >> 16));
+    f[2] = Codec<f16_tag>::widen((uint16_t)(r.y & 0xffffu)); f[3] = Codec<f16_tag>::widen((uint16_t)(r.y >> 16));
+  }
+  static __device__ __forceinline__ vec_t narrow(const float (&f)[4]) {
+    vec_t r;
+    r.x = (uint32_t)Codec<f16_tag>::narrow(f[0]) | ((uint32_t)Codec<f16_tag>::narrow(f[1]) << 16);
+    r.y = (uint32_t)Codec<f16_tag>::narrow(f[2]) | ((uint32_t)Codec<f16_tag>::narrow(f[3]) << 16);
+    return r;
+  }
+};
+
+template <class G, class A>
+__device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uint64_t gi,
+                                          uint64_t grad_elems, uint32_t i) {
+  typedef typename Codec<A>::raw_t araw_t;
+  typedef typename Codec<G>::raw_t graw_t;
+  araw_t* a = reinterpret_cast<araw_t*>(acc) + i;
+  float g = 0.0f;  // padding reads as +0 and is still added (so -0 + +0 -> +0, as F.pad + add_)
+  if (gi < grad_elems) g = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi]);
+  *a = Codec<A>::narrow(Codec<A>::widen(*a) + g);
+}
+
+// Slow path of one tile: acc[0:n] += grad[g0 : g0+n] (zero beyond grad_elems), any alignment.
+template <class G, class A>
+__device__ __forceinline__ void accum_any(uint8_t* acc, const uint8_t* grad, uint64_t g0,
+                                          uint64_t grad_elems, uint32_t n) {
+  typedef typename Quad<G>::vec_t gvec_t;
+  typedef typename Quad<A>::vec_t avec_t;
+  constexpr uint32_t kAccVecBytes = 4 * Codec<A>::kBytes;
+  const uint32_t tid = threadIdx.x;
+  uint32_t head = ((kAccVecBytes - (uint32_t)((uintptr_t)acc & (kAccVecBytes - 1))) &
+                   (kAccVecBytes - 1)) / Codec<A>::kBytes;
+  if (head > n) head = n;
+  if (tid < head) accum_one<G, A>(acc, grad, g0 + tid, grad_elems, tid);
+  const uint32_t nvec = (n - head) >> 2;
+  for (uint32_t v = tid; v < nvec; v += kThreads) {
+    const uint32_t i = head + 4 * v;
+    const uint64_t gi = g0 + i;
+    if (gi + 4 <= grad_elems) {
+      gvec_t graw;
+      __builtin_memcpy(&graw, grad + gi * Codec<G>::kBytes, sizeof(gvec_t));
+      avec_t* ap = reinterpret_cast<avec_t*>(acc + (size_t)i * Codec<A>::kBytes);
+      float gf[4], af[4];
+      Quad<G>::widen(graw, gf);
+      Quad<A>::widen(*ap, af);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
+      *ap = Quad<A>::narrow(af);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) accum_one<G, A>(acc, grad, gi + k, grad_elems, i + k);
+    }
+  }
+  const uint32_t done = head + 4 * nvec;
+  if (tid < n - done) accum_one<G, A>(acc, grad, g0 + done + tid, grad_elems, done + tid);
+}
+
+template <class G, class A>
+__global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launch) {
+  typedef typename Quad<G>::vec_t gvec_t;
+  typedef typename Quad<A>::vec_t avec_t;
+  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch, t, 0);
+    const uint64_t seg = launch.seg_elems[c.item];
+    const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
+    const uint64_t g0 = (uint64_t)c.rank * seg + in_seg;  // element index in the full gradient
+    const uint64_t grad_elems = launch.grad_elems[c.item];
+    const uint8_t* grad = launch.grad[c.item];
+    uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.acc_off[c.item] +
+                   in_seg * Codec<A>::kBytes;
+    const uint64_t left = seg - in_seg;
+    const uintptr_t gaddr = (uintptr_t)(grad + g0 * Codec<G>::kBytes);
+    if (left >= kTileElems && g0 + kTileElems <= grad_elems &&
+        (((uintptr_t)acc) & (sizeof(avec_t) - 1)) == 0 && (gaddr & (sizeof(gvec_t) - 1)) == 0) {
+      const gvec_t* gp = reinterpret_cast<const gvec_t*>(gaddr) + threadIdx.x;
+      avec_t* ap = reinterpret_cast<avec_t*>(acc) + threadIdx.x;
+      gvec_t graw[kUnroll];
+      avec_t araw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) graw[u] = __builtin_nontemporal_load(gp + u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) araw[u] = __builtin_nontemporal_load(ap + u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        float gf[4], af[4];
+        Quad<G>::widen(graw[u], gf);
+        Quad<A>::widen(araw[u], af);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
+        __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * kThreads);
+      }
+    } else {
+      accum_any<G, A>(acc, grad, g0, grad_elems, left < kTileElems ? (uint32_t)left : kTileElems);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side: arena
+// ------------------------------------------------------------------------------------------------
+constexpr uint64_t kAlign = 256;
+
+inline uint64_t round_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+struct odc_arena {
+  uint32_t world = 0;
+  int device = -1;
+  uint32_t flags = 0;
+  int n_cu = 256;
+  uint64_t bytes_per_rank = 0;
+  uint64_t rank_stride = 0;
+  uint8_t* base = nullptr;
+  std::map<uint64_t, uint64_t> live;  // offset -> size (rounded)
+  std::map<uint64_t, uint64_t> free_; // offset -> size, coalesced
+  uint64_t in_use = 0;
+  uint64_t high_water = 0;
+  std::mutex mu;
+};
+
+namespace {
+
+int check_arena(const odc_arena* a) {
+  if (!a) return fail(ODC_ERR_INVALID, "arena is NULL");
+  return ODC_OK;
+}
+
+int check_compute(odc_arena* a) {
+  if (int rc = check_arena(a)) return rc;
+  if (!a->base)
+    return fail(ODC_ERR_NO_BACKING, "arena has no device memory (created with ODC_ARENA_NO_BACKING)");
+  int cur = -1;
+  ODC_HIP_TRY(hipGetDevice(&cur));
+  if (cur != a->device) ODC_HIP_TRY(hipSetDevice(a->device));
+  return ODC_OK;
+}
+
+uint32_t grid_for(const odc_arena* a, int64_t blocks_per_cu, uint32_t n_tiles) {
+  if (blocks_per_cu <= 0) return n_tiles;
+  const uint64_t g = (uint64_t)a->n_cu * (uint64_t)blocks_per_cu;
+  return (uint32_t)std::min<uint64_t>(g, n_tiles);
+}
+
+constexpr uint64_t kMaxTilesPerLaunch = 1ull << 31;
+
+}  // namespace
+
+extern "C" {
+
+const char* odc_last_error(void) { return g_err; }
+
+int odc_abi_version(void) { return ODC_HIP_ABI_VERSION; }
+
+int odc_set_option(const char* name, int64_t value) {
+  std::lock_guard<std::mutex> lk(g_opt_mu);
+  int64_t* s = option_slot(name);
+  if (!s) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
+  if (value < 0) return fail(ODC_ERR_INVALID, "option '%s' must be >= 0", name);
+  *s = value;
+  return ODC_OK;
+}
+
+int odc_get_option(const char* name, int64_t* value) {
+  std::lock_guard<std::mutex> lk(g_opt_mu);
+  int64_t* s = option_slot(name);
+  if (!s || !value) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
+  *value = *s;
+  return ODC_OK;
+}
+
+int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flags,
+                     odc_arena** out) {
+  if (!out) return fail(ODC_ERR_INVALID, "out is NULL");
+  *out = nullptr;
+  if (world_size == 0) return fail(ODC_ERR_INVALID, "world_size must be >= 1");
+  if (bytes_per_rank == 0) return fail(ODC_ERR_INVALID, "bytes_per_rank must be > 0");
+  if (flags & ~(uint32_t)ODC_ARENA_NO_BACKING) return fail(ODC_ERR_INVALID, "unknown flags 0x%x", flags);
+  odc_arena* a = new (std::nothrow) odc_arena();
+  if (!a) return fail(ODC_ERR_NOMEM, "host allocation failed");
+  a->world = world_size;
+  a->flags = flags;
+  a->bytes_per_rank = round_up(bytes_per_rank, kAlign);
+  a->rank_stride = a->bytes_per_rank + round_up((uint64_t)g_opt.rank_stagger_bytes, kAlign);
+  if (a->rank_stride > (~0ull) / world_size) {
+    delete a;
+    return fail(ODC_ERR_INVALID, "arena size overflows 64 bits");
+  }
+  if (!(flags & ODC_ARENA_NO_BACKING)) {
+    hipError_t e = hipGetDevice(&a->device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&a->n_cu, hipDeviceAttributeMultiprocessorCount, a->device);
+    void* p = nullptr;
+    if (e == hipSuccess) e = hipMalloc(&p, a->rank_stride * world_size);
+    if (e != hipSuccess) {
+      delete a;
+      return fail(e == hipErrorOutOfMemory ? ODC_ERR_NOMEM : ODC_ERR_HIP,
+                  "creating a %u x %llu byte arena failed: %s", world_size,
+                  (unsigned long long)bytes_per_rank, hipGetErrorString(e));
+    }
+    a->base = static_cast<uint8_t*>(p);
+    if (a->n_cu <= 0) a->n_cu = 256;
+  }
+  a->free_[0] = a->bytes_per_rank;
+  *out = a;
+  return ODC_OK;
+}
+
+int odc_arena_destroy(odc_arena* a) {
+  if (int rc = check_arena(a)) return rc;
+  int rc = ODC_OK;
+  if (a->base) {
+    int cur = -1;
+    hipError_t e = hipGetDevice(&cur);
+    if (e == hipSuccess && cur != a->device) e = hipSetDevice(a->device);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipFree(a->base);
+    if (e != hipSuccess) rc = fail(ODC_ERR_HIP, "releasing the arena failed: %s", hipGetErrorString(e));
+  }
+  delete a;
+  return rc;
+}
+
+int odc_arena_alloc(odc_arena* a, uint64_t nbytes, uint64_t* offset) {
+  if (int rc = check_arena(a)) return rc;
+  if (!offset) return fail(ODC_ERR_INVALID, "offset is NULL");
+  std::lock_guard<std::mutex> lk(a->mu);
+  const uint64_t need = std::max<uint64_t>(round_up(nbytes, kAlign), kAlign);
+  if (need < nbytes) return fail(ODC_ERR_INVALID, "nbytes overflows");
+  for (auto it = a->free_.begin(); it != a->free_.end(); ++it) {  // first fit
+    if (it->second < need) continue;
+    const uint64_t off = it->first, sz = it->second;
+    a->free_.erase(it);
+    if (sz > need) a->free_[off + need] = sz - need;
+    a->live[off] = need;
+    a->in_use += need;
+    a->high_water = std::max(a->high_water, off + need);
+    *offset = off;
+    return ODC_OK;
+  }
+  return fail(ODC_ERR_NOMEM,
+              "symmetric arena exhausted: need %llu bytes per rank, %llu of %llu in use "
+              "(raise ODC_SYMMETRIC_SIZE)",
+              (unsigned long long)need, (unsigned long long)a->in_use,
+              (unsigned long long)a->bytes_per_rank);
+}
+
+int odc_arena_free(odc_arena* a, uint64_t offset) {
+  if (int rc = check_arena(a)) return rc;
+  std::lock_guard<std::mutex> lk(a->mu);
+  auto it = a->live.find(offset);
+  if (it == a->live.end())
+    return fail(ODC_ERR_NOT_FOUND, "offset %llu is not a live allocation", (unsigned long long)offset);
+  uint64_t off = it->first, sz = it->second;
+  a->live.erase(it);
+  a->in_use -= sz;
+  auto next = a->free_.lower_bound(off);
+  if (next != a->free_.end() && off + sz == next->first) {  // merge with the block after
+    sz += next->second;
+    next = a->free_.erase(next);
+  }
+  if (next != a->free_.begin()) {  // merge with the block before
+    auto prev = std::prev(next);
+    if (prev->first + prev->second == off) {
+      prev->second += sz;
+      return ODC_OK;
+    }
+  }
+  a->free_[off] = sz;
+  return ODC_OK;
+}
+
+int odc_arena_reset(odc_arena* a) {
+  if (int rc = check_arena(a)) return rc;
+  std::lock_guard<std::mutex> lk(a->mu);
+  a->live.clear();
+  a->free_.clear();
+  a->free_[0] = a->bytes_per_rank;
+  a->in_use = 0;
+  return ODC_OK;
+}
+
+int odc_arena_get_info(const odc_arena* a, odc_arena_info* info) {
+  if (int rc = check_arena(a)) return rc;
+  if (!info) return fail(ODC_ERR_INVALID, "info is NULL");
+  odc_arena* m = const_cast<odc_arena*>(a);
+  std::lock_guard<std::mutex> lk(m->mu);
+  info->world_size = a->world;
+  info->device = a->base ? a->device : -1;
+  info->flags = a->flags;
+  info->n_allocations = (uint32_t)a->live.size();
+  info->bytes_per_rank = a->bytes_per_rank;
+  info->rank_stride = a->rank_stride;
+  info->base = (uint64_t)(uintptr_t)a->base;
+  info->bytes_in_use = a->in_use;
+  info->high_water = a->high_water;
+  return ODC_OK;
+}
+
+void* odc_arena_ptr(const odc_arena* a, uint32_t rank, uint64_t offset) {
+  if (!a || !a->base || rank >= a->world || offset > a->bytes_per_rank) {
+    fail(ODC_ERR_INVALID, "odc_arena_ptr: bad arena, rank %u or offset %llu", rank,
+         (unsigned long long)offset);
+    return nullptr;
+  }
+  return a->base + (uint64_t)rank * a->rank_stride + offset;
+}
+
+int odc_arena_locate(const odc_arena* a, const void* ptr, uint32_t* rank, uint64_t* alloc_offset,
+                     uint64_t* inner) {
+  if (int rc = check_arena(a)) return rc;
+  if (!a->base) return fail(ODC_ERR_NO_BACKING, "arena has no device memory");
+  const uint8_t* p = static_cast<const uint8_t*>(ptr);
+  if (p < a->base || p >= a->base + a->rank_stride * a->world)
+    return fail(ODC_ERR_NOT_FOUND, "pointer %p is outside the arena", ptr);
+  const uint64_t d = (uint64_t)(p - a->base);
+  const uint32_t r = (uint32_t)(d / a->rank_stride);
+  const uint64_t off = d - (uint64_t)r * a->rank_stride;
+  odc_arena* m = const_cast<odc_arena*>(a);
+  std::lock_guard<std::mutex> lk(m->mu);
+  auto it = a->live.upper_bound(off);
+  if (it == a->live.begin()) return fail(ODC_ERR_NOT_FOUND, "pointer %p is not in a live allocation", ptr);
+  --it;
+  if (off >= it->first + it->second)
+    return fail(ODC_ERR_NOT_FOUND, "pointer %p is not in a live allocation", ptr);
+  if (rank) *rank = r;
+  if (alloc_offset) *alloc_offset = it->first;
+  if (inner) *inner = off - it->first;
+  return ODC_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// launches
+// ------------------------------------------------------------------------------------------------
+int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uint32_t first_rank,
+               void* stream) {
+  if (int rc = check_compute(a)) return rc;
+  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
+  if (first_rank >= a->world)
+    return fail(ODC_ERR_INVALID, "first_rank %u >= world size %u", first_rank, a->world);
+  for (uint32_t i = 0; i < n_items; ++i) {
+    const odc_gather_item& it = items[i];
+    if (it.shard_bytes == 0) continue;
+    if (!it.dst) return fail(ODC_ERR_INVALID, "item %u: dst is NULL", i);
+    if (it.src_offset > a->bytes_per_rank || it.shard_bytes > a->bytes_per_rank - it.src_offset)
+      return fail(ODC_ERR_INVALID, "item %u: [%llu, +%llu) leaves the %llu byte rank region", i,
+                  (unsigned long long)it.src_offset, (unsigned long long)it.shard_bytes,
+                  (unsigned long long)a->bytes_per_rank);
+    const uint8_t* d0 = static_cast<const uint8_t*>(it.dst);
+    const uint8_t* d1 = d0 + it.shard_bytes * a->world;
+    const uint8_t* s0 = a->base + it.src_offset;
+    const uint8_t* s1 = a->base + (uint64_t)(a->world - 1) * a->rank_stride + it.src_offset + it.shard_bytes;
+    if (d0 < s1 && s0 < d1) {
+      // dst lies somewhere inside the arena span: refuse only a true overlap with a shard read
+      for (uint32_t r = 0; r < a->world; ++r) {
+        const uint8_t* rs0 = a->base + (uint64_t)r * a->rank_stride + it.src_offset;
+        if (d0 < rs0 + it.shard_bytes && rs0 < d1)
+          return fail(ODC_ERR_INVALID, "item %u: dst overlaps rank %u's shard", i, r);
+      }
+    }
+  }
+  const Options opt = g_opt;
+  uint32_t i = 0;
+  while (i < n_items) {
+    GatherLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.world = a->world;
+    L.first_rank = first_rank;
+    L.rank_major = opt.rank_major ? 1u : 0u;
+    uint32_t n = 0;
+    uint64_t tiles = 0;
+    for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
+      if (items[i].shard_bytes == 0) continue;
+      const uint64_t tps = (items[i].shard_bytes + kTileBytes - 1) / kTileBytes;
+      if (tps * a->world >= kMaxTilesPerLaunch)
+        return fail(ODC_ERR_INVALID, "item %u: shard of %llu bytes is too large for one launch", i,
+                    (unsigned long long)items[i].shard_bytes);
+      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
+      L.tile_prefix[n] = (uint32_t)tiles;
+      L.tiles_per_seg[n] = (uint32_t)tps;
+      L.dst[n] = static_cast<uint8_t*>(items[i].dst);
+      L.src_off[n] = items[i].src_offset;
+      L.seg_bytes[n] = items[i].shard_bytes;
+      tiles += tps * a->world;
+      ++n;
+    }
+    if (n == 0) continue;
+    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
+    L.n_items = n;
+    L.n_tiles = (uint32_t)tiles;
+    const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.n_tiles);
+    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* stream) {
+  if (int rc = check_compute(a)) return rc;
+  if (n_spans && !spans) return fail(ODC_ERR_INVALID, "spans is NULL");
+  for (uint32_t i = 0; i < n_spans; ++i) {
+    if (spans[i].offset > a->bytes_per_rank || spans[i].nbytes > a->bytes_per_rank - spans[i].offset)
+      return fail(ODC_ERR_INVALID, "span %u: [%llu, +%llu) leaves the %llu byte rank region", i,
+                  (unsigned long long)spans[i].offset, (unsigned long long)spans[i].nbytes,
+                  (unsigned long long)a->bytes_per_rank);
+  }
+  const Options opt = g_opt;
+  uint32_t i = 0;
+  while (i < n_spans) {
+    ClearLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.world = a->world;
+    L.rank_major = opt.rank_major ? 1u : 0u;
+    uint32_t n = 0;
+    uint64_t tiles = 0;
+    for (; i < n_spans && n < (uint32_t)kMaxItems; ++i) {
+      if (spans[i].nbytes == 0) continue;
+      const uint64_t tps = (spans[i].nbytes + kTileBytes - 1) / kTileBytes;
+      if (tps * a->world >= kMaxTilesPerLaunch)
+        return fail(ODC_ERR_INVALID, "span %u: %llu bytes is too large for one launch", i,
+                    (unsigned long long)spans[i].nbytes);
+      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
+      L.tile_prefix[n] = (uint32_t)tiles;
+      L.tiles_per_seg[n] = (uint32_t)tps;
+      L.off[n] = spans[i].offset;
+      L.seg_bytes[n] = spans[i].nbytes;
+      tiles += tps * a->world;
+      ++n;
+    }
+    if (n == 0) continue;
+    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
+    L.n_items = n;
+    L.n_tiles = (uint32_t)tiles;
+    const uint32_t grid = grid_for(a, opt.clear_blocks_per_cu, L.n_tiles);
+    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+int dtype_bytes(int dt) {
+  switch (dt) {
+    case ODC_DTYPE_BF16: return 2;
+    case ODC_DTYPE_F16: return 2;
+    case ODC_DTYPE_F32: return 4;
+    default: return 0;
+  }
+}
+
+typedef void (*accum_fn)(const AccumLaunch);
+
+accum_fn pick_accum(int g, int a) {
+#define ODC_PAIR(GE, GT, AE, AT) if (g == GE && a == AE) return accum_kernel<GT, AT>;
+  ODC_PAIR(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_F32, f32_tag)
+  ODC_PAIR(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F32, f32_tag)
+  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F32, f32_tag)
+  ODC_PAIR(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_BF16, bf16_tag)
+  ODC_PAIR(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F16, f16_tag)
+  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_BF16, bf16_tag)
+  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F16, f16_tag)
+#undef ODC_PAIR
+  return nullptr;
+}
+
+}  // namespace
+
+extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
+                                      int grad_dtype, int acc_dtype, void* stream) {
+  if (int rc = check_compute(a)) return rc;
+  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
+  const int gb = dtype_bytes(grad_dtype), ab = dtype_bytes(acc_dtype);
+  if (!gb || !ab) return fail(ODC_ERR_INVALID, "unknown dtype code (grad %d, acc %d)", grad_dtype, acc_dtype);
+  const accum_fn kernel = pick_accum(grad_dtype, acc_dtype);
+  if (!kernel)
+    return fail(ODC_ERR_UNSUPPORTED, "scatter-accumulate of grad dtype %d into acc dtype %d is not implemented",
+                grad_dtype, acc_dtype);
+  for (uint32_t i = 0; i < n_items; ++i) {
+    const odc_accum_item& it = items[i];
+    if (it.shard_elems == 0) {
+      if (it.grad_elems) return fail(ODC_ERR_INVALID, "item %u: grad_elems > 0 with shard_elems == 0", i);
+      continue;
+    }
+    if (it.shard_elems > a->bytes_per_rank / ab)
+      return fail(ODC_ERR_INVALID, "item %u: shard of %llu elements exceeds the rank region", i,
+                  (unsigned long long)it.shard_elems);
+    if (it.acc_offset % ab)
+      return fail(ODC_ERR_INVALID, "item %u: acc_offset %llu is not aligned to the accumulation dtype", i,
+                  (unsigned long long)it.acc_offset);
+    if (it.acc_offset > a->bytes_per_rank || it.shard_elems * ab > a->bytes_per_rank - it.acc_offset)
+      return fail(ODC_ERR_INVALID, "item %u: accumulation [%llu, +%llu) leaves the %llu byte rank region", i,
+                  (unsigned long long)it.acc_offset, (unsigned long long)(it.shard_elems * ab),
+                  (unsigned long long)a->bytes_per_rank);
+    if (it.grad_elems > it.shard_elems * a->world)
+      return fail(ODC_ERR_INVALID, "item %u: grad_elems %llu > world_size * shard_elems = %llu", i,
+                  (unsigned long long)it.grad_elems, (unsigned long long)(it.shard_elems * a->world));
+    if (it.grad_elems && !it.grad) return fail(ODC_ERR_INVALID, "item %u: grad is NULL", i);
+    if ((uintptr_t)it.grad % gb)
+      return fail(ODC_ERR_INVALID, "item %u: grad pointer is not aligned to the gradient dtype", i);
+  }
+  const Options opt = g_opt;
+  uint32_t i = 0;
+  while (i < n_items) {
+    AccumLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.world = a->world;
+    L.rank_major = opt.rank_major ? 1u : 0u;
+    uint32_t n = 0;
+    uint64_t tiles = 0;
+    for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
+      if (items[i].shard_elems == 0) continue;
+      const uint64_t tps = (items[i].shard_elems + kTileElems - 1) / kTileElems;
+      if (tps * a->world >= kMaxTilesPerLaunch)
+        return fail(ODC_ERR_INVALID, "item %u: shard of %llu elements is too large for one launch", i,
+                    (unsigned long long)items[i].shard_elems);
+      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
+      L.tile_prefix[n] = (uint32_t)tiles;
+      L.tiles_per_seg[n] = (uint32_t)tps;
+      L.grad[n] = static_cast<const uint8_t*>(items[i].grad);
+      L.grad_elems[n] = items[i].grad_elems;
+      L.acc_off[n] = items[i].acc_offset;
+      L.seg_elems[n] = items[i].shard_elems;
+      tiles += tps * a->world;
+      ++n;
+    }
+    if (n == 0) continue;
+    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
+    L.n_items = n;
+    L.n_tiles = (uint32_t)tiles;
+    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.n_tiles);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}

@@ -1,0 +1,178 @@
+"""On-demand scatter-accumulate: a full gradient is added, chunk r into rank r's accumulation
+buffer, by one fused HIP launch.
+
+Mirror of ``odc/primitives/scatter_accumulate.py`` (``ReductionService``, :494-749). In the
+reference the caller copies chunk r into a staging buffer on rank r (:649-669), rings a doorbell
+(:671-688) and a watcher process on rank r performs ``acc[start:start+size].add_(buf[:size])``
+(:369-395). With every rank's accumulation in one HBM the owner is the caller, so staging,
+doorbells and the watcher collapse into ``odc_scatter_accumulate`` (include/odc_hip.h): one read
+of the gradient, one read-modify-write of the accumulations.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import logging
+from typing import Sequence
+
+import torch
+
+from odc_amd import _native
+from odc_amd.primitives.utils import (
+    BufferSplitter,
+    SymmBufferRegistry,
+    get_comm_stream,
+    get_rank,
+    get_world,
+    group_size,
+    native_dtype,
+)
+
+logger = logging.getLogger(__name__)
+
+
+class ReductionService:
+    def __init__(self, accumulation_dtype=None):
+        self.accumulations = []  # index -> key (tensors come from the registry, per rank)
+        self.accumulation_indices = {}
+        self.accumulation_dtype = accumulation_dtype
+        self.dispatched_tasks = 0
+        self.buffer_splitter = BufferSplitter()
+
+    # -- registration ---------------------------------------------------------------------
+    @staticmethod
+    def _acc_key(key):
+        return f"rs_accumulation_{key}"
+
+    def register(self, key, output_tensor_shape, grad_dtype, reduction_dtype, pg):
+        """Allocate the zero-initialised symmetric accumulation ``rs_accumulation_{key}``
+        (scatter_accumulate.py:551-555; the watcher zeroes it at :357-362). No staging buffers
+        are created: the fused kernel reads the caller's gradient directly."""
+        assert len(output_tensor_shape) == 1
+        assert key not in self.accumulation_indices
+        native_dtype(grad_dtype), native_dtype(reduction_dtype)  # reject unsupported dtypes early
+        registry = SymmBufferRegistry.get_instance()
+        accumulation_key = self._acc_key(key)
+        assert not registry.has_key(accumulation_key)
+        registry.allocate_symm_buffer(accumulation_key, tuple(output_tensor_shape), reduction_dtype)
+        self.accumulation_indices[key] = len(self.accumulations)
+        self.accumulations.append(key)
+        self._clear_keys([key])
+
+    def _clear_keys(self, keys):
+        if not keys:
+            return
+        registry = SymmBufferRegistry.get_instance()
+        spans = (_native.Span * len(keys))()
+        for i, key in enumerate(keys):
+            offset, shape, dtype = registry.offsets[self._acc_key(key)]
+            spans[i].offset = offset
+            spans[i].nbytes = shape[0] * dtype.itemsize
+        comm = get_comm_stream()
+        comm.wait_stream(torch.cuda.current_stream())
+        _native.check(
+            _native.load().odc_clear(
+                get_world().arena.handle, spans, len(spans), ctypes.c_void_p(comm.cuda_stream)
+            )
+        )
+        torch.cuda.current_stream().wait_stream(comm)
+
+    def clear_accumulations(self):
+        """Zero every registered accumulation of EVERY virtual rank in one launch
+        (``acc.fill_(0)`` per key and per process in the reference, :585-587). Idempotent, so
+        each virtual rank may call it; like there, no rank may have started the minibatch's
+        scatter-accumulates before the last clear."""
+        self._clear_keys(self.accumulations)
+
+    # -- the primitive ----------------------------------------------------------------------
+    def infer_output_shape(self, input_tensor, pg):
+        assert len(input_tensor.shape) == 1
+        assert input_tensor.shape[0] % group_size(pg) == 0
+        return (input_tensor.shape[0] // group_size(pg),)
+
+    def scatter_accumulate(self, key, input_tensor, pg) -> None:
+        """``acc_r[key] += input_tensor.view(W, -1)[r]`` for every rank r."""
+        self.scatter_accumulate_multi([key], [input_tensor], pg)
+
+    def scatter_accumulate_multi(
+        self, keys: Sequence, input_tensors: Sequence[torch.Tensor], pg, valid_numels=None
+    ) -> None:
+        """Multi-tensor form: all (key, gradient) pairs in ONE launch (per 32 pairs).
+
+        ``valid_numels[i]``, when given, says that only the first so many elements of the
+        padded gradient i exist at ``input_tensors[i]``; the rest read as +0 (the ``F.pad`` of
+        ``odc/fsdp/fsdp1.py:25-38`` without materialising it). Then ``input_tensors[i]`` may be
+        shorter than W * shard and the shard size comes from the registered accumulation.
+        """
+        assert len(keys) == len(input_tensors)
+        world = get_world()
+        W = group_size(pg)
+        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+        registry = SymmBufferRegistry.get_instance()
+        grad_dtype = input_tensors[0].dtype
+        items = (_native.AccumItem * len(keys))()
+        acc_dtype = None
+        for i, (key, grad) in enumerate(zip(keys, input_tensors)):
+            assert grad.is_cuda, "scatter-accumulate runs on the GPU only"
+            assert grad.dtype == grad_dtype, "one launch takes one gradient dtype"
+            assert grad.is_contiguous()
+            if valid_numels is None:
+                shard_shape = self.infer_output_shape(grad, pg)
+                valid = grad.numel()
+            else:
+                assert key in self.accumulation_indices, "padded form needs a registered key"
+                shard_shape = registry.offsets[self._acc_key(key)][1]
+                valid = int(valid_numels[i])
+                assert valid <= grad.numel() and valid <= W * shard_shape[0]
+            if key not in self.accumulation_indices:
+                accum_dtype = (
+                    self.accumulation_dtype if self.accumulation_dtype is not None else grad.dtype
+                )
+                self.register(key, shard_shape, grad.dtype, accum_dtype, pg)
+            offset, acc_shape, this_acc_dtype = registry.offsets[self._acc_key(key)]
+            assert tuple(acc_shape) == tuple(
+                shard_shape
+            ), f"key {key}: registered shard {acc_shape}, gradient implies {shard_shape}"
+            assert acc_dtype in (None, this_acc_dtype), "one launch takes one accumulation dtype"
+            acc_dtype = this_acc_dtype
+            items[i].grad = grad.data_ptr()
+            items[i].grad_elems = valid
+            items[i].acc_offset = offset
+            items[i].shard_elems = shard_shape[0]
+
+        comm = get_comm_stream()
+        comm.wait_stream(torch.cuda.current_stream())
+        _native.check(
+            _native.load().odc_scatter_accumulate(
+                world.arena.handle,
+                items,
+                len(items),
+                native_dtype(grad_dtype),
+                native_dtype(acc_dtype),
+                ctypes.c_void_p(comm.cuda_stream),
+            )
+        )
+        self.dispatched_tasks += len(items)
+        torch.cuda.current_stream().wait_stream(comm)
+
+    # -- results ----------------------------------------------------------------------------
+    def get_accumulation(self, key):
+        """The calling rank's live accumulation buffer (callers mutate it in place,
+        ``odc/fsdp/fsdp2.py:846-847``)."""
+        if key not in self.accumulation_indices:
+            raise KeyError(key)
+        return SymmBufferRegistry.get_instance().get_symm_buffer(self._acc_key(key))
+
+    def get_peer_accumulations(self, key):
+        """All W ranks' accumulation buffers for ``key`` (virtual-world convenience)."""
+        return SymmBufferRegistry.get_instance().peer_tensors[self._acc_key(key)]
+
+    def sync(self, pg=None):
+        """Block until every dispatched add has landed (:734-743: the reference counts tasks
+        across ranks and waits for its watcher; here all adds are on the comm stream)."""
+        get_comm_stream().synchronize()
+        self.dispatched_tasks = 0
+
+    def stop(self):
+        if torch.cuda.is_available():
+            get_comm_stream().synchronize()

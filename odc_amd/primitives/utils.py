@@ -1,0 +1,458 @@
+"""Symmetric memory for W virtual ranks on one MI355X.
+
+Host-side mirror of ``odc/primitives/utils.py``: the same names (``init_nvshmem``,
+``finalize_distributed``, ``SymmBufferRegistry``, ``BufferSplitter``, ``get_comm_stream``,
+``get_local_world_size``) with the NVSHMEM symmetric heap replaced by the arena of
+``libodc_hip.so``: one ``hipMalloc`` cut into W rank regions, where one byte offset names the
+same buffer in every region. A *virtual rank* is one of those regions; the process plays any of
+them (``set_rank`` / ``virtual_rank``) the way one process per GPU plays its rank in the
+reference.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import ctypes
+import logging
+import math
+import os
+from functools import reduce
+from typing import List, Optional
+
+import torch
+
+from odc_amd import _native
+
+logger = logging.getLogger(__name__)
+
+_SIZE_SUFFIX = {"K": 2**10, "M": 2**20, "G": 2**30, "T": 2**40}
+
+
+def parse_size(text) -> int:
+    """'30G', '5000000000', '512M' -> bytes (the forms NVSHMEM_SYMMETRIC_SIZE takes,
+    launch.sh:135, README.md:53-57)."""
+    if isinstance(text, int):
+        return text
+    s = str(text).strip().upper().rstrip("B")
+    if s and s[-1] in _SIZE_SUFFIX:
+        return int(float(s[:-1]) * _SIZE_SUFFIX[s[-1]])
+    return int(s)
+
+
+_TORCH_TO_NATIVE = {
+    torch.bfloat16: _native.DTYPE_BF16,
+    torch.float16: _native.DTYPE_F16,
+    torch.float32: _native.DTYPE_F32,
+}
+
+
+def native_dtype(dtype: torch.dtype) -> int:
+    try:
+        return _TORCH_TO_NATIVE[dtype]
+    except KeyError:
+        raise TypeError(f"scatter-accumulate supports bf16/fp16/fp32, not {dtype}") from None
+
+
+class VirtualGroup:
+    """Stands in for a ``torch.distributed.ProcessGroup`` wherever the reference takes ``pg``:
+    W virtual ranks living in one HBM. Only ``size()`` and ``rank()`` are ever asked of it."""
+
+    def __init__(self, world_size: int):
+        self._world_size = int(world_size)
+
+    def size(self) -> int:
+        return self._world_size
+
+    def rank(self) -> int:
+        return get_rank()
+
+    def __repr__(self):
+        return f"VirtualGroup(world_size={self._world_size})"
+
+
+def group_size(pg) -> int:
+    """``torch.distributed.get_world_size(pg)`` for real and virtual groups; None = the world."""
+    if pg is None:
+        return get_world().world_size
+    return pg.size()
+
+
+class _ArenaMemory:
+    """Exposes the arena to torch through ``__cuda_array_interface__`` (zero copy, non-owning)."""
+
+    def __init__(self, ptr: int, nbytes: int):
+        self.__cuda_array_interface__ = {
+            "shape": (nbytes,),
+            "typestr": "|u1",
+            "data": (ptr, False),
+            "version": 2,
+            "strides": None,
+        }
+
+
+class SymmetricArena:
+    """Python handle of one ``odc_arena`` (include/odc_hip.h)."""
+
+    def __init__(self, world_size: int, bytes_per_rank: int, backing: bool = True):
+        self._lib = _native.load()
+        self._handle = ctypes.c_void_p()
+        flags = _native.ODC_ARENA_DEVICE if backing else _native.ODC_ARENA_NO_BACKING
+        _native.check(
+            self._lib.odc_arena_create(
+                int(world_size), int(bytes_per_rank), flags, ctypes.byref(self._handle)
+            )
+        )
+        info = self.info()
+        self.world_size = info.world_size
+        self.bytes_per_rank = info.bytes_per_rank
+        self.rank_stride = info.rank_stride
+        self.base = info.base
+        self.device = info.device
+        self._bytes = None
+        if backing:
+            mem = _ArenaMemory(self.base, self.rank_stride * self.world_size)
+            self._bytes = torch.as_tensor(mem, device=torch.device("cuda", self.device))
+            assert self._bytes.data_ptr() == self.base, "torch did not alias the arena"
+
+    @property
+    def handle(self):
+        if self._handle is None or not self._handle.value:
+            raise RuntimeError("the symmetric arena has been finalized")
+        return self._handle
+
+    def info(self) -> _native.ArenaInfo:
+        info = _native.ArenaInfo()
+        _native.check(self._lib.odc_arena_get_info(self.handle, ctypes.byref(info)))
+        return info
+
+    def alloc(self, nbytes: int) -> int:
+        off = ctypes.c_uint64()
+        _native.check(self._lib.odc_arena_alloc(self.handle, int(nbytes), ctypes.byref(off)))
+        return off.value
+
+    def free(self, offset: int) -> None:
+        _native.check(self._lib.odc_arena_free(self.handle, int(offset)))
+
+    def reset(self) -> None:
+        _native.check(self._lib.odc_arena_reset(self.handle))
+
+    def ptr(self, rank: int, offset: int) -> int:
+        p = self._lib.odc_arena_ptr(self.handle, int(rank), int(offset))
+        if not p:
+            raise _native.OdcNativeError(
+                _native.ODC_ERR_INVALID, self._lib.odc_last_error().decode()
+            )
+        return p
+
+    def locate(self, ptr: int):
+        """device address -> (rank, allocation offset, distance into the allocation)."""
+        rank, off, inner = ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_uint64()
+        _native.check(
+            self._lib.odc_arena_locate(
+                self.handle, ctypes.c_void_p(ptr), ctypes.byref(rank), ctypes.byref(off),
+                ctypes.byref(inner),
+            )
+        )
+        return rank.value, off.value, inner.value
+
+    def view(self, rank: int, offset: int, shape, dtype: torch.dtype) -> torch.Tensor:
+        """Non-owning tensor over rank ``rank``'s copy of the buffer at ``offset``."""
+        if self._bytes is None:
+            raise RuntimeError("a bookkeeping-only arena has no memory to view")
+        numel = reduce(lambda x, y: x * y, shape, 1)
+        nbytes = numel * dtype.itemsize
+        if not 0 <= rank < self.world_size or offset + nbytes > self.bytes_per_rank:
+            raise ValueError(f"view of rank {rank} [{offset}, +{nbytes}) leaves the rank region")
+        start = rank * self.rank_stride + offset
+        return self._bytes[start : start + nbytes].view(dtype).view(tuple(shape))
+
+    def destroy(self) -> None:
+        if self._handle is not None and self._handle.value:
+            self._bytes = None
+            handle, self._handle = self._handle, None
+            _native.check(self._lib.odc_arena_destroy(handle))
+
+
+class _VirtualWorld:
+    def __init__(self, arena: SymmetricArena):
+        self.arena = arena
+        self.world_size = arena.world_size
+        self.rank = 0
+        self.group = VirtualGroup(self.world_size)
+
+
+_world: Optional[_VirtualWorld] = None
+
+
+def get_world() -> _VirtualWorld:
+    if _world is None:
+        raise RuntimeError("init_nvshmem() has not been called: there is no symmetric arena")
+    return _world
+
+
+def is_initialized() -> bool:
+    return _world is not None
+
+
+def init_nvshmem(world_size: Optional[int] = None, symmetric_size=None):
+    """Create the symmetric arena (the name is the reference's, ``utils.py:18-49``, where it boots
+    NVSHMEM over the global process group).
+
+    ``world_size``: number of virtual ranks W; default ``$ODC_VIRTUAL_WORLD_SIZE``, else
+    ``get_local_world_size()``. ``symmetric_size``: bytes per rank; default
+    ``$ODC_SYMMETRIC_SIZE``, else ``$NVSHMEM_SYMMETRIC_SIZE`` (the reference's knob,
+    ``launch.sh:135``), else 1 GiB. Returns the world's ``VirtualGroup``.
+    """
+    global _world
+    if _world is not None:
+        raise RuntimeError("init_nvshmem() called twice without finalize_distributed()")
+    if world_size is None:
+        env = os.environ.get("ODC_VIRTUAL_WORLD_SIZE")
+        world_size = int(env) if env else get_local_world_size()
+    if symmetric_size is None:
+        symmetric_size = os.environ.get(
+            "ODC_SYMMETRIC_SIZE", os.environ.get("NVSHMEM_SYMMETRIC_SIZE", "1G")
+        )
+    nbytes = parse_size(symmetric_size)
+    if not torch.cuda.is_available():
+        raise RuntimeError("init_nvshmem() needs a GPU: the symmetric arena lives in HBM")
+    _world = _VirtualWorld(SymmetricArena(world_size, nbytes))
+    logger.info(f"symmetric arena: {world_size} ranks x {nbytes} bytes")
+    return _world.group
+
+
+def finalize_distributed():
+    """Release the arena (``utils.py:84-85``). Tensors handed out by the registry dangle after
+    this, exactly as NVSHMEM tensors do after ``nvshmem.core.finalize``."""
+    global _world, stream
+    if _world is not None:
+        if hasattr(SymmBufferRegistry, "_instance"):
+            SymmBufferRegistry._instance._forget()
+        _world.arena.destroy()
+        _world = None
+    stream = None
+
+
+def get_rank() -> int:
+    """The virtual rank this process currently plays (``torch.distributed.get_rank()`` there)."""
+    return get_world().rank
+
+
+def get_world_size() -> int:
+    return get_world().world_size
+
+
+def set_rank(rank: int) -> None:
+    world = get_world()
+    if not 0 <= rank < world.world_size:
+        raise ValueError(f"rank {rank} outside [0, {world.world_size})")
+    world.rank = int(rank)
+
+
+@contextlib.contextmanager
+def virtual_rank(rank: int):
+    """``with virtual_rank(r):`` — act as rank r, then return to the previous rank."""
+    prev = get_rank()
+    set_rank(rank)
+    try:
+        yield
+    finally:
+        set_rank(prev)
+
+
+class SymmBufferRegistry:
+    """name -> symmetric buffer, ``utils.py:88-172``.
+
+    ``local_tensor[key]`` is the current rank's view at the time of the lookup;
+    ``peer_tensors[key]`` are all W views. Both alias arena memory and own nothing.
+    """
+
+    def __init__(self, arena=None, rank_fn=None):
+        # arena/rank_fn default to the process-wide virtual world; passing them gives a
+        # registry of its own (used to exercise the bookkeeping without a GPU)
+        self._arena = arena
+        self._rank_fn = rank_fn
+        self.offsets = {}  # key -> (offset, shape, dtype)
+        self.local_tensor_to_keys = {}  # data_ptr of any rank's view -> key
+        self.updated = set()  # (key, rank)
+        self.peer_tensors = {}
+        self.allocations = []
+
+    @property
+    def arena(self):
+        return self._arena if self._arena is not None else get_world().arena
+
+    @classmethod
+    def get_instance(cls):
+        if not hasattr(cls, "_instance"):
+            cls._instance = SymmBufferRegistry()
+        return cls._instance
+
+    @property
+    def local_tensor(self):
+        """key -> the current rank's tensor (a fresh dict; the reference's attribute of the
+        same name, read by ``fsdp2.get_symm_buffer_memory_breakdown``)."""
+        rank = self._rank()
+        return {k: peers[rank] for k, peers in self.peer_tensors.items()}
+
+    def _rank(self) -> int:
+        return self._rank_fn() if self._rank_fn is not None else get_rank()
+
+    # we'll mark all symm buffers dirty; the next update_symm_buffer copies again
+    def flush(self):
+        self.updated.clear()
+
+    def update_symm_buffer(self, buffer_key, values):
+        values = values.contiguous()
+        if buffer_key not in self.peer_tensors:
+            self.allocate_symm_buffer(buffer_key, values.shape, values.dtype)
+        rank = self._rank()
+        local = self.peer_tensors[buffer_key][rank]
+        if (buffer_key, rank) not in self.updated:
+            self.updated.add((buffer_key, rank))
+            local.copy_(values)
+            # the reference barriers here so that peers see the shard; with one process the
+            # copy is ordered before later work on the same stream, and gather's stream join
+            # (comm_stream.wait_stream(current)) orders it before any read.
+        return local
+
+    @classmethod
+    def set_nvshmem_flag(cls, tensor):
+        tensor._odc_is_nvshmem = True
+
+    @classmethod
+    def is_nvshmem_tensor(cls, tensor):
+        return hasattr(tensor, "_odc_is_nvshmem") and tensor._odc_is_nvshmem
+
+    def allocate_symm_buffer(self, key, shape, dtype):
+        assert key not in self.peer_tensors
+        arena = self.arena
+        shape = tuple(shape)
+        numel = reduce(lambda x, y: x * y, shape, 1)
+        offset = arena.alloc(numel * dtype.itemsize)
+        peers = [arena.view(r, offset, shape, dtype) for r in range(arena.world_size)]
+        for t in peers:
+            self.set_nvshmem_flag(t)
+            self.local_tensor_to_keys[t.data_ptr()] = key
+        self.allocations.append(peers[0])
+        self.offsets[key] = (offset, shape, dtype)
+        self.peer_tensors[key] = peers
+        local = peers[self._rank()]
+        logger.info(
+            f"Rank {self._rank()} create tensor {key} with shape {shape} and dtype {dtype} "
+            f"and ptr {local.data_ptr()}"
+        )
+        return local
+
+    def has_key(self, key):
+        return key in self.peer_tensors
+
+    def get_or_create_symm_buffer(self, key, shape, dtype):
+        if self.has_key(key):
+            return self.peer_tensors[key][self._rank()]
+        return self.allocate_symm_buffer(key, shape, dtype)
+
+    def get_symm_buffer(self, key):
+        if self.has_key(key):
+            return self.peer_tensors[key][self._rank()]
+        raise ValueError(f"Symm buffer {key} not found")
+
+    def get_peer_tensors(self, local_tensor) -> List[torch.Tensor]:
+        buffer_key = self.local_tensor_to_keys[local_tensor.data_ptr()]
+        return self.peer_tensors[buffer_key]
+
+    def get_offset(self, key) -> int:
+        """Symmetric byte offset of a registered buffer (what the kernels take)."""
+        return self.offsets[key][0]
+
+    def symmetric_offset_of(self, tensor: torch.Tensor) -> int:
+        """Symmetric byte offset of ``tensor``, which must be (a contiguous view into) a
+        registered buffer of any rank. Exact buffer starts resolve through the data_ptr map
+        (``utils.py:158-161``); inner views through ``odc_arena_locate``."""
+        key = self.local_tensor_to_keys.get(tensor.data_ptr())
+        if key is not None:
+            return self.offsets[key][0]
+        if not tensor.is_cuda:
+            raise ValueError("tensor is not in the symmetric arena")
+        try:
+            _rank, off, inner = self.arena.locate(tensor.data_ptr())
+        except _native.OdcNativeError as e:
+            raise ValueError(f"tensor is not in the symmetric arena: {e.message}") from None
+        return off + inner
+
+    def _forget(self):
+        self.offsets.clear()
+        self.local_tensor_to_keys.clear()
+        self.updated.clear()
+        self.peer_tensors.clear()
+        self.allocations.clear()
+
+    def finalize(self):
+        arena = self.arena if (self._arena is not None or is_initialized()) else None
+        if arena is not None:
+            if torch.cuda.is_available():
+                torch.cuda.synchronize()
+            for offset, _shape, _dtype in self.offsets.values():
+                arena.free(offset)
+        self._forget()
+
+    def memory_allocated(self):
+        return sum(t.nbytes for t in self.allocations)
+
+
+def get_local_world_size():
+    """Ranks per node (``utils.py:195-199``); here it is also the default number of virtual ranks."""
+    if _world is not None:
+        return _world.world_size
+    if "RAY_LOCAL_WORLD_SIZE" in os.environ:
+        return int(os.environ["RAY_LOCAL_WORLD_SIZE"])
+    else:
+        return int(os.environ["LOCAL_WORLD_SIZE"])
+
+
+stream = None
+
+
+def get_comm_stream():
+    """One side stream for all primitive launches (``utils.py:205-209``), default priority."""
+    global stream
+    if stream is None:
+        stream = torch.cuda.Stream()
+    return stream
+
+
+class BufferSplitter:
+    """Sub-request sizing rule of the reference (``utils.py:212-242``), in elements.
+
+    ``ODC_MAX_BUFFER_SIZE`` (default 64 Mi elements; <= 0 turns splitting off) caps the staging
+    buffer of a whole request; one rank's slice of it is rounded up to 64 elements. Callers size
+    buffers with these numbers, so the closed forms are kept; the fused kernels here never
+    split a request, and results do not depend on the setting.
+    """
+
+    DEFAULT_MAX_BUFFER_SIZE = 64 * 1024 * 1024
+
+    def __init__(self):
+        self.round_data_size = 2**6
+
+    def get_max_global_buffer_size(self) -> int:
+        return int(os.environ.get("ODC_MAX_BUFFER_SIZE", self.DEFAULT_MAX_BUFFER_SIZE))
+
+    def round_to_data_size(self, size: int) -> int:
+        q = self.round_data_size
+        return -(-size // q) * q
+
+    def get_global_buffer_size(self, original_buffer_shape) -> int:
+        numel = math.prod(original_buffer_shape)
+        cap = self.get_max_global_buffer_size()
+        return numel if cap <= 0 else min(cap, numel)
+
+    def get_local_buffer_size(self, original_buffer_shape, world_size) -> int:
+        numel = math.prod(original_buffer_shape)
+        cap = self.get_max_global_buffer_size()
+        if cap > 0:
+            assert (
+                cap % world_size == 0
+            ), f"ODC_MAX_BUFFER_SIZE: {cap} % world_size: {world_size} != 0"
+            numel = min(cap // world_size, numel)
+        return self.round_to_data_size(numel)

@@ -1,0 +1,180 @@
+"""GPU parity of the two primitives against the CPU oracle, through the Python mirror of the
+reference API (which calls the C ABI of libodc_hip.so). Bit-exact: gather is a byte copy;
+scatter-accumulate does one IEEE fp32 add per element per call, in call order."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    """Integer view for bit-exact comparison (NaN-safe)."""
+    return t.contiguous().view({1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+
+
+def assert_bit_equal(got: torch.Tensor, want: torch.Tensor, what=""):
+    got, want = got.cpu(), want.cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype, what
+    if not torch.equal(bits(got), bits(want)):
+        bad = (bits(got) != bits(want)).nonzero().flatten()
+        i = int(bad[0])
+        raise AssertionError(
+            f"{what}: {bad.numel()} of {got.numel()} elements differ; first at {i}: "
+            f"got {got.flatten()[i].item()!r} want {want.flatten()[i].item()!r}"
+        )
+
+
+def services():
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry
+
+    return GatherService(), ReductionService(accumulation_dtype=torch.float32), SymmBufferRegistry.get_instance()
+
+
+def put_shards(registry, key, shards, group):
+    """Each virtual rank publishes its shard, as each process does in the reference
+    (examples/all_gather.py:82-84)."""
+    from odc_amd import virtual_rank
+
+    local = None
+    for r, s in enumerate(shards):
+        with virtual_rank(r):
+            t = registry.update_symm_buffer(key, s.cuda())
+            if r == 0:
+                local = t
+    return local
+
+
+def test_gather_known_answer_pattern(make_world):
+    """examples/all_gather.py:80-84,121-125: tensor i on rank r is filled with i + 2r; block r of
+    the gathered tensor must equal 2r + i exactly (int64 there and here)."""
+    W, size, cnt = 8, 1 << 16, 5
+    group = make_world(W, 64 << 20)
+    gather, _, registry = services()
+    for i in range(cnt):
+        shards = [torch.full((size,), i + 2 * r, dtype=torch.int64) for r in range(W)]
+        src = put_shards(registry, i, shards, group)
+        dst = torch.empty(size * W, dtype=torch.int64, device="cuda")
+        gather.gather_into_tensor(dst, src, group)
+        for r in range(W):
+            assert torch.eq(dst[r * size : (r + 1) * size], 2 * r + i).all()
+
+
+def test_config1_plumbing(make_world):
+    """W=4, one flat bf16 param of 4 Mi elements N(0, 0.02) seed 0 in 4 equal shards, gathered;
+    then 4 microbatches of bf16 grads N(0, 1e-3) scatter-accumulated into zeroed fp32 shards."""
+    W, N, M = 4, 4_194_304, 4
+    g = torch.Generator().manual_seed(0)
+    param = (torch.randn(N, generator=g) * 0.02).bfloat16()
+    grads = [(torch.randn(N, generator=g) * 1e-3).bfloat16() for _ in range(M)]
+    shards = list(param.view(W, -1))
+
+    group = make_world(W, 64 << 20)
+    gather, reduction, registry = services()
+    src = put_shards(registry, "flat", shards, group)
+    out = torch.empty(N, dtype=torch.bfloat16, device="cuda")
+    gather.gather_into_tensor(out, src, group)
+    assert_bit_equal(out, oracle.gather(shards), "gather")
+    assert_bit_equal(out, param, "gather vs original")
+
+    want = [torch.zeros(N // W, dtype=torch.float32) for _ in range(W)]
+    reduction.clear_accumulations()
+    for m in range(M):
+        reduction.scatter_accumulate("flat", grads[m].cuda(), group)
+        oracle.scatter_accumulate(want, grads[m])
+    reduction.sync(group)
+    for r, acc in enumerate(reduction.get_peer_accumulations("flat")):
+        assert_bit_equal(acc, want[r], f"accumulation of rank {r}")
+    # clear brings every rank back to +0.0
+    reduction.clear_accumulations()
+    reduction.sync(group)
+    for acc in reduction.get_peer_accumulations("flat"):
+        assert_bit_equal(acc, torch.zeros(N // W), "cleared accumulation")
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 5, 8, 12, 64])
+@pytest.mark.parametrize("S", [0, 1, 7, 63, 64, 65, 4095, 4096, 4097, 16384 + 3, 100_003])
+def test_gather_any_shard_size(make_world, W, S):
+    """Byte copy at every alignment: odd shard sizes put block r of the output at odd offsets."""
+    group = make_world(W, 4 << 20)
+    gather, _, registry = services()
+    g = torch.Generator().manual_seed(W * 1000 + S)
+    shards = [torch.randint(-32768, 32767, (S,), generator=g, dtype=torch.int16) for _ in range(W)]
+    src = put_shards(registry, "p", shards, group)
+    # sentinels on both sides of the destination catch writes outside [0, W*S)
+    pad = 64
+    buf = torch.full((W * S + 2 * pad,), -999, dtype=torch.int16, device="cuda")
+    dst = buf[pad : pad + W * S]
+    from odc_amd import virtual_rank
+
+    with virtual_rank(W - 1):  # rotation start must not matter (gather.py:122)
+        gather.gather_into_tensor(dst, registry.get_symm_buffer("p"), group)
+    assert_bit_equal(dst, oracle.gather(shards), f"W={W} S={S}")
+    assert (buf[:pad] == -999).all() and (buf[pad + W * S :] == -999).all()
+
+
+@pytest.mark.parametrize("grad_dtype,acc_dtype", [
+    (torch.bfloat16, torch.float32),
+    (torch.float32, torch.float32),
+    (torch.float16, torch.float32),
+    (torch.bfloat16, torch.bfloat16),
+    (torch.float16, torch.float16),
+])
+@pytest.mark.parametrize("W,S", [(1, 5), (4, 1), (8, 4096), (8, 4099), (12, 33_337), (3, 70_001)])
+def test_scatter_accumulate_dtypes_and_sizes(make_world, grad_dtype, acc_dtype, W, S):
+    from odc_amd import ReductionService
+
+    group = make_world(W, 4 << 20)
+    reduction = ReductionService(accumulation_dtype=acc_dtype)
+    g = torch.Generator().manual_seed(S)
+    want = [torch.zeros(S, dtype=acc_dtype) for _ in range(W)]
+    for m in range(3):
+        grad = torch.randn(W * S, generator=g).to(grad_dtype)
+        reduction.scatter_accumulate(7, grad.cuda(), group)
+        oracle.scatter_accumulate(want, grad)
+    reduction.sync(group)
+    for r, acc in enumerate(reduction.get_peer_accumulations(7)):
+        assert_bit_equal(acc, want[r], f"{grad_dtype}->{acc_dtype} W={W} S={S} rank {r}")
+
+
+def test_scatter_accumulate_special_values(make_world):
+    """Signed zero (+0 + -0 = +0), denormals, infinities, NaN propagation, bf16 extremes."""
+    W = 4
+    group = make_world(W, 4 << 20)
+    from odc_amd import ReductionService
+
+    reduction = ReductionService(accumulation_dtype=torch.float32)
+    # every bf16 bit pattern once, as the gradient
+    all_bf16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    assert all_bf16.numel() % W == 0
+    want = [torch.zeros(all_bf16.numel() // W) for _ in range(W)]
+    for _ in range(2):
+        reduction.scatter_accumulate("all", all_bf16.cuda(), group)
+        oracle.scatter_accumulate(want, all_bf16)
+    reduction.sync(group)
+    for r, acc in enumerate(reduction.get_peer_accumulations("all")):
+        got, w = acc.cpu(), want[r]
+        nan = torch.isnan(w)
+        assert torch.equal(torch.isnan(got), nan)
+        assert_bit_equal(got[~nan], w[~nan], f"rank {r}")
+    # -0 gradients into a cleared (+0) accumulation give +0, not -0
+    neg0 = torch.full((W * 8,), -0.0).bfloat16()
+    reduction.scatter_accumulate("z", neg0.cuda(), group)
+    reduction.sync(group)
+    for acc in reduction.get_peer_accumulations("z"):
+        assert not torch.signbit(acc.cpu()).any()
+    # fp32 denormals survive (no flush to zero)
+    tiny = torch.full((W * 8,), 1e-41, dtype=torch.float32)
+    reduction.scatter_accumulate("d", tiny.cuda(), group)
+    reduction.scatter_accumulate("d", tiny.cuda(), group)
+    reduction.sync(group)
+    wantd = [torch.zeros(8) for _ in range(W)]
+    oracle.scatter_accumulate(wantd, tiny)
+    oracle.scatter_accumulate(wantd, tiny)
+    for r, acc in enumerate(reduction.get_peer_accumulations("d")):
+        assert_bit_equal(acc, wantd[r], "denormal")
+        assert (acc.cpu() != 0).all()
