@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the ODC hot path on one MI355X: gather + scatter-accumulate over a Llama-3-8B
+decoder layer sharded over W=8 virtual ranks.
+
+One step = one microbatch of the path over the whole layer:
+    gather            all 9 parameters, bf16, W shards -> full tensors      (one launch, 4N bytes)
+    scatter-accumulate all 9 bf16 gradients into the W fp32 accumulations   (one launch, 10N bytes)
+Every 8th step starts a new minibatch and first clears the accumulations (inside the timed
+region; its 4N written bytes are NOT counted in the numerator).
+
+Prints ONE JSON line (see README / DESIGN for the fields).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+MICROBATCHES = 8
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE and
+# WRITE_SIZE runs, scaled by a torch copy kernel of known size); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--world-size", type=int, default=8, help="virtual ranks W")
+    ap.add_argument("--layout", choices=["per-param", "flat"], default="per-param",
+                    help="9 per-parameter shards in one multi-tensor launch, or one flat shard")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="libodc_hip launch knob, e.g. accum_blocks_per_cu=4")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: W virtual ranks share one MI355X and nothing here uses a "
+              "second GPU. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import odc_amd
+    from odc_amd import _native
+    from odc_amd.primitives.utils import get_comm_stream
+    from odc_amd.workloads import llama3_8b_layer_shapes, numel
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    for opt in args.option:
+        name, value = opt.split("=")
+        _native.set_option(name, int(value))
+
+    W = args.world_size
+    shapes = llama3_8b_layer_shapes()
+    if args.layout == "flat":
+        shapes = [("flat", (sum(numel(s) for _, s in shapes),))]
+    numels = [numel(s) for _, s in shapes]
+    assert all(n % W == 0 for n in numels)
+    N = sum(numels)
+    per_rank = sum((n // W) * 6 + 512 for n in numels) + (1 << 20)
+    group = odc_amd.init_nvshmem(world_size=W, symmetric_size=per_rank)
+    registry = odc_amd.SymmBufferRegistry.get_instance()
+    gather = odc_amd.GatherService()
+    reduction = odc_amd.ReductionService(accumulation_dtype=torch.float32)
+
+    # synthetic data, generated on the device and mirrored to the host for the oracle
+    dev_gen = torch.Generator(device="cuda").manual_seed(0)
+    params = [(torch.randn(n, generator=dev_gen, device="cuda") * 0.02).bfloat16() for n in numels]
+    grads = [[(torch.randn(n, generator=dev_gen, device="cuda") * 1e-3).bfloat16() for n in numels]
+             for _ in range(MICROBATCHES)]
+    keys = [name for name, _ in shapes]
+    shard_locals = []
+    for key, p in zip(keys, params):
+        for r in range(W):
+            with odc_amd.virtual_rank(r):
+                t = registry.update_symm_buffer(key, p.view(W, -1)[r])
+        shard_locals.append(registry.get_symm_buffer(key))
+    outs = [torch.empty_like(p) for p in params]
+    # register the accumulations up front (lazy registration is not part of a steady-state step)
+    for key, n in zip(keys, numels):
+        reduction.register(key, (n // W,), torch.bfloat16, torch.float32, group)
+    torch.cuda.synchronize()
+
+    comm = get_comm_stream()
+    gather_events, accum_events, clear_events = [], [], []
+
+    def step(i, record):
+        m = i % MICROBATCHES
+        if m == 0:
+            if record:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(comm)
+            reduction.clear_accumulations()
+            if record:
+                e1.record(comm)
+                clear_events.append((e0, e1))
+        if record:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(comm)
+        gather.gather_into_tensors(outs, shard_locals, group)
+        if record:
+            e1.record(comm)
+            gather_events.append((e0, e1))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(comm)
+        reduction.scatter_accumulate_multi(keys, grads[m], group)
+        if record:
+            e1.record(comm)
+            accum_events.append((e0, e1))
+
+    # ---- parity + CPU baseline: one full minibatch against the oracle -------------------------
+    cpu_baseline = None
+    parity = None
+    if not args.no_verify or not args.no_cpu_baseline:
+        from oracle import odc_oracle as oracle
+
+        for i in range(MICROBATCHES):
+            step(i, record=False)
+        reduction.sync(group)
+        host_params = [p.cpu() for p in params]
+        host_grads = [[g.cpu() for g in mb] for mb in grads]
+        host_outs = [torch.empty_like(p) for p in host_params]
+        host_accs = [[torch.zeros(n // W, dtype=torch.float32) for _ in range(W)] for n in numels]
+        host_shards = [list(p.view(W, -1)) for p in host_params]
+        t0 = time.perf_counter()
+        for m in range(MICROBATCHES):
+            for o, sh in zip(host_outs, host_shards):
+                oracle.gather_into_tensor(o, sh)
+            for accs, g in zip(host_accs, host_grads[m]):
+                oracle.scatter_accumulate(accs, g)
+        cpu_s = time.perf_counter() - t0
+        cpu_baseline = {
+            "value": round(MICROBATCHES * 14 * N / cpu_s / 1e9, 3),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{MICROBATCHES} microbatches of the same layer (gather + scatter-accumulate), "
+                      f"torch CPU oracle, {cpu_s:.2f} s",
+        }
+        if not args.no_verify:
+            ok = True
+            for o, ho in zip(outs, host_outs):
+                ok &= torch.equal(o.cpu().view(torch.int16), ho.view(torch.int16))
+            for key, accs in zip(keys, host_accs):
+                for r, acc in enumerate(reduction.get_peer_accumulations(key)):
+                    ok &= torch.equal(acc.cpu().view(torch.int32), accs[r].view(torch.int32))
+            parity = bool(ok)
+            if not ok:
+                print("PARITY FAILURE: GPU results differ from the CPU oracle", file=sys.stderr)
+        del host_params, host_grads, host_outs, host_accs, host_shards
+
+    # ---- timed region -----------------------------------------------------------------------
+    for i in range(args.warmup):
+        step(i, record=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, record=True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    if args.calibrate:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
+
+    def mean_ms(pairs):
+        return statistics.fmean(a.elapsed_time(b) for a, b in pairs) if pairs else None
+
+    g_ms, a_ms, c_ms = mean_ms(gather_events), mean_ms(accum_events), mean_ms(clear_events)
+    accum_gbps = 10 * N / (a_ms * 1e-3) / 1e9
+    gather_gbps = 4 * N / (g_ms * 1e-3) / 1e9
+    value = args.steps * 14 * N / elapsed / 1e9
+    workload = (f"cfg2: Llama-3-8B decoder layer ({N} bf16 params, {len(keys)} tensors, "
+                f"{args.layout}), W={W} virtual shards, {MICROBATCHES} microbatches per minibatch")
+    result = {
+        "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for gather + scatter-accum, 8B layer, W=8",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": workload, "world_size": W, "elements": N,
+                   "bytes_per_step": 14 * N, "layout": args.layout},
+        "frac_of_peak": round(value / HBM_PEAK_GBPS, 4),
+        "roofline": {
+            "kernel": "accum_kernel<bf16,f32> (scatter-accumulate)",
+            "bound": "hbm",
+            "achieved": round(accum_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(accum_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("accum", args.layout, W)),
+            "algorithmic_bytes": 10 * N,
+            "avg_launch_ms": round(a_ms, 5),
+        },
+        "roofline_gather": {
+            "kernel": "gather_kernel",
+            "bound": "hbm",
+            "achieved": round(gather_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gather_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("gather", args.layout, W)),
+            "algorithmic_bytes": 4 * N,
+            "avg_launch_ms": round(g_ms, 5),
+        },
+        "clear": {"avg_launch_ms": round(c_ms, 5) if c_ms else None,
+                  "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},
+        "cpu_baseline": cpu_baseline,
+        "parity_vs_oracle": parity,
+    }
+    print(json.dumps(result))
+    torch.cuda.synchronize()
+    registry.finalize()
+    odc_amd.finalize_distributed()
+    if parity is False:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

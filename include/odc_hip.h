@@ -160,9 +160,10 @@ const char* odc_last_error(void);
 int odc_abi_version(void);
 
 /* Launch-shape knobs, for measurement. Names: "gather_blocks_per_cu", "accum_blocks_per_cu",
- * "clear_blocks_per_cu" (0 = one block per tile, no grid-stride loop), "rank_major" (1 = walk a
- * rank's whole shard before the next rank, 0 = interleave ranks tile by tile). Unknown names
- * return ODC_ERR_INVALID. Results never depend on these. */
+ * "clear_blocks_per_cu" (0 = one block per tile, no grid-stride loop), "rank_major" (gather and
+ * scatter-accumulate: 1 = walk a rank's whole shard before the next rank, 0 = interleave ranks
+ * tile by tile), "rank_stagger_bytes" (extra distance between rank regions, read when an arena
+ * is created). Unknown names return ODC_ERR_INVALID. Results never depend on these. */
 int odc_set_option(const char* name, int64_t value);
 int odc_get_option(const char* name, int64_t* value);
 

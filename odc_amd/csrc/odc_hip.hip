@@ -57,9 +57,11 @@ int fail(int code, const char* fmt, ...) {
 // options
 // ------------------------------------------------------------------------------------------------
 struct Options {
-  int64_t gather_blocks_per_cu = 8;
-  int64_t accum_blocks_per_cu = 8;
-  int64_t clear_blocks_per_cu = 8;
+  // measured on MI355X over a Llama-3-8B layer: gather peaks at 2 workgroups per CU, the
+  // read-modify-write at 1, the pure-write clear with one workgroup per tile
+  int64_t gather_blocks_per_cu = 2;
+  int64_t accum_blocks_per_cu = 1;
+  int64_t clear_blocks_per_cu = 0;
   int64_t rank_major = 1;
   int64_t rank_stagger_bytes = 0;
 };
@@ -717,7 +719,7 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
     L.base = a->base;
     L.rank_stride = a->rank_stride;
     L.world = a->world;
-    L.rank_major = opt.rank_major ? 1u : 0u;
+    L.rank_major = 0u;  // a write-only stream runs fastest with the ranks interleaved
     uint32_t n = 0;
     uint64_t tiles = 0;
     for (; i < n_spans && n < (uint32_t)kMaxItems; ++i) {

@@ -12,14 +12,13 @@ import ctypes
 import logging
 from typing import Sequence
 
-import torch
 from torch import Tensor
 
 from odc_amd import _native
 from odc_amd.primitives.utils import (
     BufferSplitter,
     SymmBufferRegistry,
-    get_comm_stream,
+    comm_stream_section,
     get_rank,
     get_world,
     group_size,
@@ -63,11 +62,35 @@ class GatherService:
             items[i].src_offset = registry.symmetric_offset_of(inp)
             items[i].shard_bytes = inp.numel() * inp.element_size()
 
-        comm = get_comm_stream()
-        comm.wait_stream(torch.cuda.current_stream())
-        _native.check(
-            _native.load().odc_gather(
-                world.arena.handle, items, len(pairs), get_rank(), ctypes.c_void_p(comm.cuda_stream)
+        with comm_stream_section() as comm:
+            _native.check(
+                _native.load().odc_gather(
+                    world.arena.handle, items, len(pairs), get_rank(),
+                    ctypes.c_void_p(comm.cuda_stream),
+                )
             )
-        )
-        torch.cuda.current_stream().wait_stream(comm)
+
+    def gather_slices(
+        self,
+        output_tensors: Sequence[Tensor],
+        input_tensor: Tensor,
+        slice_offsets: Sequence[int],
+        slice_numels: Sequence[int],
+        pg,
+    ) -> None:
+        """Gather slices of ONE symmetric buffer straight into separate outputs, in one launch:
+        ``output_i.view(W, -1)[r] = rank r's input_tensor[off_i : off_i + n_i]``.
+
+        With the FSDP2 group layout (``odc/fsdp/fsdp2.py:146-196``: the group buffer is the
+        concatenation of every parameter's padded shard) this is ``gather_into_tensor`` followed
+        by ``split_with_sizes_copy(dim=1)`` (``fsdp2.py:378-401``) without the intermediate
+        ``[W, sum n_i]`` buffer.
+        """
+        assert len(output_tensors) == len(slice_offsets) == len(slice_numels)
+        assert input_tensor.is_cuda and input_tensor.is_contiguous()
+        es = input_tensor.element_size()
+        slices = []
+        for off, n in zip(slice_offsets, slice_numels):
+            assert 0 <= off and off + n <= input_tensor.numel(), "slice leaves the buffer"
+            slices.append(input_tensor.view(-1)[off : off + n])
+        self.gather_into_tensors(list(output_tensors), slices, pg)

@@ -21,6 +21,7 @@ from odc_amd import _native
 from odc_amd.primitives.utils import (
     BufferSplitter,
     SymmBufferRegistry,
+    comm_stream_section,
     get_comm_stream,
     get_rank,
     get_world,
@@ -68,14 +69,12 @@ class ReductionService:
             offset, shape, dtype = registry.offsets[self._acc_key(key)]
             spans[i].offset = offset
             spans[i].nbytes = shape[0] * dtype.itemsize
-        comm = get_comm_stream()
-        comm.wait_stream(torch.cuda.current_stream())
-        _native.check(
-            _native.load().odc_clear(
-                get_world().arena.handle, spans, len(spans), ctypes.c_void_p(comm.cuda_stream)
+        with comm_stream_section() as comm:
+            _native.check(
+                _native.load().odc_clear(
+                    get_world().arena.handle, spans, len(spans), ctypes.c_void_p(comm.cuda_stream)
+                )
             )
-        )
-        torch.cuda.current_stream().wait_stream(comm)
 
     def clear_accumulations(self):
         """Zero every registered accumulation of EVERY virtual rank in one launch
@@ -140,20 +139,72 @@ class ReductionService:
             items[i].acc_offset = offset
             items[i].shard_elems = shard_shape[0]
 
-        comm = get_comm_stream()
-        comm.wait_stream(torch.cuda.current_stream())
-        _native.check(
-            _native.load().odc_scatter_accumulate(
-                world.arena.handle,
-                items,
-                len(items),
-                native_dtype(grad_dtype),
-                native_dtype(acc_dtype),
-                ctypes.c_void_p(comm.cuda_stream),
+        with comm_stream_section() as comm:
+            _native.check(
+                _native.load().odc_scatter_accumulate(
+                    world.arena.handle,
+                    items,
+                    len(items),
+                    native_dtype(grad_dtype),
+                    native_dtype(acc_dtype),
+                    ctypes.c_void_p(comm.cuda_stream),
+                )
             )
-        )
         self.dispatched_tasks += len(items)
-        torch.cuda.current_stream().wait_stream(comm)
+
+    def scatter_accumulate_slices(
+        self,
+        key,
+        input_tensors: Sequence[torch.Tensor],
+        slice_offsets: Sequence[int],
+        slice_numels: Sequence[int],
+        pg,
+        accumulation_numel: int = None,
+        accumulation_dtype=None,
+    ) -> None:
+        """Accumulate several gradients into slices of ONE accumulation, in one launch:
+        ``acc_r[key][off_i : off_i + n_i] += pad0(input_i).view(W, n_i)[r]``, where ``input_i``
+        holds at most ``W * n_i`` elements and what is missing reads as +0.
+
+        With the FSDP2 group layout this is ``torch._chunk_cat`` (``odc/fsdp/fsdp2.py:671-682``)
+        followed by ``scatter_accumulate`` (``fsdp2.py:708-710``) without the intermediate
+        ``[W, sum n_i]`` reduce-scatter input. The key is registered on first use with
+        ``accumulation_numel`` elements (default: the end of the last slice).
+        """
+        assert len(input_tensors) == len(slice_offsets) == len(slice_numels)
+        world = get_world()
+        W = group_size(pg)
+        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+        registry = SymmBufferRegistry.get_instance()
+        grad_dtype = input_tensors[0].dtype
+        if key not in self.accumulation_indices:
+            total = accumulation_numel
+            if total is None:
+                total = max(o + n for o, n in zip(slice_offsets, slice_numels))
+            accum_dtype = accumulation_dtype or self.accumulation_dtype or grad_dtype
+            self.register(key, (total,), grad_dtype, accum_dtype, pg)
+        offset, acc_shape, acc_dtype = registry.offsets[self._acc_key(key)]
+        items = (_native.AccumItem * len(input_tensors))()
+        for i, (grad, off, n) in enumerate(zip(input_tensors, slice_offsets, slice_numels)):
+            assert grad.is_cuda and grad.is_contiguous() and grad.dtype == grad_dtype
+            assert 0 <= off and off + n <= acc_shape[0], "slice leaves the accumulation"
+            assert grad.numel() <= W * n, f"gradient {i} has {grad.numel()} > {W} * {n} elements"
+            items[i].grad = grad.data_ptr()
+            items[i].grad_elems = grad.numel()
+            items[i].acc_offset = offset + off * acc_dtype.itemsize
+            items[i].shard_elems = n
+        with comm_stream_section() as comm:
+            _native.check(
+                _native.load().odc_scatter_accumulate(
+                    world.arena.handle,
+                    items,
+                    len(items),
+                    native_dtype(grad_dtype),
+                    native_dtype(acc_dtype),
+                    ctypes.c_void_p(comm.cuda_stream),
+                )
+            )
+        self.dispatched_tasks += 1
 
     # -- results ----------------------------------------------------------------------------
     def get_accumulation(self, key):

@@ -421,6 +421,21 @@ def get_comm_stream():
     return stream
 
 
+@contextlib.contextmanager
+def comm_stream_section():
+    """Run the body's launches on the comm stream, joined with the current stream on both
+    sides (``gather.py:114,176``; ``scatter_accumulate.py:636-640,725-727``). When the caller
+    already runs on the comm stream there is nothing to join."""
+    comm = get_comm_stream()
+    current = torch.cuda.current_stream()
+    if current == comm:
+        yield comm
+        return
+    comm.wait_stream(current)
+    yield comm
+    current.wait_stream(comm)
+
+
 class BufferSplitter:
     """Sub-request sizing rule of the reference (``utils.py:212-242``), in elements.
 

@@ -1,0 +1,115 @@
+"""The symmetric arena and registry on the GPU, through the C ABI."""
+
+import ctypes
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def test_symmetric_offsets_and_views(make_world):
+    from odc_amd import SymmBufferRegistry, virtual_rank
+    from odc_amd.primitives import utils
+
+    W = 5
+    make_world(W, 1 << 20)
+    arena = utils.get_world().arena
+    reg = SymmBufferRegistry.get_instance()
+    a = reg.allocate_symm_buffer("a", (1000,), torch.float32)
+    b = reg.allocate_symm_buffer("b", (3, 5), torch.bfloat16)
+    assert reg.is_nvshmem_tensor(a) and a.shape == (1000,) and b.shape == (3, 5)
+    peers = reg.get_peer_tensors(a)
+    assert len(peers) == W and peers[0].data_ptr() == a.data_ptr()
+    stride = arena.info().rank_stride
+    for r, t in enumerate(peers):
+        assert t.data_ptr() == arena.ptr(r, reg.get_offset("a")) == a.data_ptr() + r * stride
+        assert arena.locate(t.data_ptr() + 40) == (r, reg.get_offset("a"), 40)
+    with virtual_rank(3):
+        assert reg.get_symm_buffer("a").data_ptr() == peers[3].data_ptr()
+        assert reg.get_peer_tensors(reg.get_symm_buffer("a")) is peers
+    # writes through one rank's view land only in that rank's region
+    for r, t in enumerate(peers):
+        t.fill_(float(r))
+    for r, t in enumerate(peers):
+        assert (t.cpu() == r).all()
+    with pytest.raises(AssertionError):
+        reg.allocate_symm_buffer("a", (1,), torch.float32)  # utils.py:127
+    with pytest.raises(ValueError):
+        reg.get_symm_buffer("missing")  # utils.py:153-156
+    assert reg.memory_allocated() == 1000 * 4 + 15 * 2
+
+
+def test_update_symm_buffer_copies_once_until_flush(make_world):
+    """utils.py:103-116."""
+    from odc_amd import SymmBufferRegistry
+
+    make_world(2, 1 << 20)
+    reg = SymmBufferRegistry.get_instance()
+    t = reg.update_symm_buffer(7, torch.arange(10.0).cuda())
+    assert_bit_equal(t, torch.arange(10.0), "first update copies")
+    t2 = reg.update_symm_buffer(7, torch.zeros(10).cuda())
+    assert t2.data_ptr() == t.data_ptr()
+    assert_bit_equal(t2, torch.arange(10.0), "second update is a no-op")
+    reg.flush()
+    assert_bit_equal(reg.update_symm_buffer(7, torch.ones(10).cuda()), torch.ones(10), "after flush")
+
+
+def test_arena_exhaustion_and_bad_arguments(make_world):
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry, _native
+    from odc_amd.primitives import utils
+
+    group = make_world(4, 1 << 16)
+    reg = SymmBufferRegistry.get_instance()
+    with pytest.raises(_native.OdcNativeError) as e:
+        reg.allocate_symm_buffer("big", (1 << 20,), torch.float32)
+    assert e.value.code == _native.ODC_ERR_NOMEM and "ODC_SYMMETRIC_SIZE" in str(e.value)
+    src = reg.allocate_symm_buffer("s", (64,), torch.bfloat16)
+    gather = GatherService()
+    with pytest.raises(AssertionError):  # output numel must be W * shard numel
+        gather.gather_into_tensor(torch.empty(100, dtype=torch.bfloat16, device="cuda"), src, group)
+    with pytest.raises(ValueError):  # input must live in the arena
+        gather.gather_into_tensor(torch.empty(256, dtype=torch.bfloat16, device="cuda"),
+                                  torch.empty(64, dtype=torch.bfloat16, device="cuda"), group)
+    red = ReductionService(accumulation_dtype=torch.float32)
+    with pytest.raises(AssertionError):  # shape[0] % W (scatter_accumulate.py:589-592)
+        red.scatter_accumulate("k", torch.zeros(10, dtype=torch.bfloat16, device="cuda"), group)
+    with pytest.raises(TypeError):
+        red.scatter_accumulate("k", torch.zeros(8, dtype=torch.int32, device="cuda"), group)
+    # raw C ABI: offsets outside the rank region are refused, nothing is launched
+    lib = _native.load()
+    arena = utils.get_world().arena
+    item = (_native.GatherItem * 1)()
+    item[0].dst = src.data_ptr()
+    item[0].src_offset = 1 << 16
+    item[0].shard_bytes = 64
+    assert lib.odc_gather(arena.handle, item, 1, 0, None) == _native.ODC_ERR_INVALID
+    assert lib.odc_gather(arena.handle, item, 1, 9, None) == _native.ODC_ERR_INVALID  # first_rank >= W
+    # dst overlapping a shard it reads
+    item[0].src_offset = reg.get_offset("s")
+    item[0].shard_bytes = 32
+    assert lib.odc_gather(arena.handle, item, 1, 0, None) == _native.ODC_ERR_INVALID
+    assert b"overlaps" in lib.odc_last_error()
+    torch.cuda.synchronize()
+
+
+def test_gather_from_inner_view_and_multi_item(make_world):
+    """A shard that is a slice of a larger symmetric buffer resolves through odc_arena_locate."""
+    from odc_amd import GatherService, SymmBufferRegistry, virtual_rank
+
+    W = 3
+    group = make_world(W, 1 << 20)
+    reg = SymmBufferRegistry.get_instance()
+    reg.allocate_symm_buffer("g", (1000,), torch.int32)
+    for r in range(W):
+        with virtual_rank(r):
+            reg.get_symm_buffer("g").copy_(torch.arange(1000, dtype=torch.int32) + 10_000 * r)
+    local = reg.get_symm_buffer("g")
+    out_a = torch.empty(W * 100, dtype=torch.int32, device="cuda")
+    out_b = torch.empty(W * 7, dtype=torch.int32, device="cuda")
+    GatherService().gather_into_tensors([out_a, out_b], [local[50:150], local[993:1000]], group)
+    for r in range(W):
+        assert_bit_equal(out_a[r * 100 : (r + 1) * 100], torch.arange(50, 150, dtype=torch.int32) + 10_000 * r)
+        assert_bit_equal(out_b[r * 7 : (r + 1) * 7], torch.arange(993, 1000, dtype=torch.int32) + 10_000 * r)

@@ -1,0 +1,118 @@
+"""The benchmark configurations at their full sizes (2-4) against the CPU oracle.
+
+Inputs are drawn on the device from a seeded generator and mirrored to the host, so the HIP path
+and the oracle see identical bits; the oracle handles these sizes in seconds."""
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal, device_randn_bf16
+from odc_amd.workloads import llama3_8b_layer_shapes, numel, shard_numel, uneven_flat_numels
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _services():
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry
+
+    return GatherService(), ReductionService(accumulation_dtype=torch.float32), SymmBufferRegistry.get_instance()
+
+
+def _run_layer(make_world, W, layout, microbatches):
+    shapes = llama3_8b_layer_shapes()
+    numels = [numel(s) for _, s in shapes]
+    if layout == "flat":
+        numels = [sum(numels)]
+    N = sum(numels)
+    assert N == 218_112_000
+    per_rank = sum((n // W) * 6 + 512 for n in numels) + (1 << 20)
+    group = make_world(W, per_rank)
+    gather, reduction, registry = _services()
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    params = [device_randn_bf16(n, gen, 0.02) for n in numels]
+    keys = list(range(len(numels)))
+    from odc_amd import virtual_rank
+
+    for key, p in zip(keys, params):
+        for r in range(W):
+            with virtual_rank(r):
+                registry.update_symm_buffer(key, p.view(W, -1)[r])
+    outs = [torch.full_like(p, float("nan")) for p in params]
+    gather.gather_into_tensors(outs, [registry.get_symm_buffer(k) for k in keys], group)
+    for o, p in zip(outs, params):  # gather of equal shards of p is p itself
+        assert torch.equal(o.view(torch.int16), p.view(torch.int16))
+        host = p.cpu()
+        assert_bit_equal(o, oracle.gather(list(host.view(W, -1))), "gather vs oracle")
+    del outs
+
+    want = [[torch.zeros(n // W) for _ in range(W)] for n in numels]
+    for _ in range(microbatches):
+        grads = [device_randn_bf16(n, gen, 1e-3) for n in numels]
+        reduction.scatter_accumulate_multi(keys, grads, group)
+        for accs, g in zip(want, grads):
+            oracle.scatter_accumulate(accs, g.cpu())
+    reduction.sync(group)
+    for key, accs in zip(keys, want):
+        for r, acc in enumerate(reduction.get_peer_accumulations(key)):
+            assert_bit_equal(acc, accs[r], f"W={W} {layout} key {key} rank {r}")
+
+
+@pytest.mark.parametrize("layout", ["per-param", "flat"])
+def test_config2_llama_layer_w8(make_world, layout):
+    """Llama-3-8B decoder layer, W=8: 9 per-parameter shards in one multi-tensor launch, and the
+    same 218 112 000 elements as one flat shard of 27 264 000."""
+    _run_layer(make_world, 8, layout, microbatches=3)
+
+
+@pytest.mark.parametrize("layout", ["per-param", "flat"])
+def test_config4_small_chunks_w64(make_world, layout):
+    """The same layer at W=64: shards from 917 504 elements down to the 64-element (128 B)
+    slices of the two norm vectors."""
+    _run_layer(make_world, 64, layout, microbatches=2)
+
+
+def test_config3_uneven_padded_w12(make_world):
+    """40 flat parameters with numel not divisible by W=12; shard = ceil(numel/12), the last
+    rank's tail zero padded (FSDP1 rule); all 40 gathered by ONE fused launch; gradients are
+    passed unpadded and the kernel supplies the +0 tail."""
+    W, M = 12, 4
+    numels = uneven_flat_numels(40, W)
+    assert len(numels) == 40 and all(n % W for n in numels)
+    shard = [shard_numel(n, W) for n in numels]
+    per_rank = sum(s * 6 + 512 for s in shard) + (1 << 20)
+    group = make_world(W, per_rank)
+    gather, reduction, registry = _services()
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    from odc_amd import virtual_rank
+
+    host_params, locals_ = [], []
+    for i, n in enumerate(numels):
+        p = device_randn_bf16(n, gen, 0.02).cpu()
+        host_params.append(p)
+        for r in range(W):
+            with virtual_rank(r):
+                registry.update_symm_buffer(i, oracle.fsdp1_get_shard(p, r, W).cuda())
+        locals_.append(registry.get_symm_buffer(i))
+    outs = [torch.full((W * s,), float("nan"), dtype=torch.bfloat16, device="cuda") for s in shard]
+    gather.gather_into_tensors(outs, locals_, group)  # 40 items -> 2 launches of <= 32
+    for i, (o, p) in enumerate(zip(outs, host_params)):
+        want = oracle.gather([oracle.fsdp1_get_shard(p, r, W) for r in range(W)])
+        assert_bit_equal(o, want, f"param {i} (numel {numels[i]})")
+        assert_bit_equal(o[: numels[i]], p, f"param {i} unpadded prefix")
+        assert not o[numels[i] :].cpu().float().abs().any(), "padding must be zero"
+    del outs
+
+    keys = list(range(len(numels)))
+    for k, s in zip(keys, shard):
+        reduction.register(k, (s,), torch.bfloat16, torch.float32, group)
+    want = [[torch.zeros(s) for _ in range(W)] for s in shard]
+    for _ in range(M):
+        grads = [device_randn_bf16(n, gen, 1e-3) for n in numels]
+        reduction.scatter_accumulate_multi(keys, grads, group, valid_numels=numels)
+        for accs, g in zip(want, grads):
+            oracle.scatter_accumulate(accs, oracle.fsdp1_pad_grad(g.cpu(), W))
+    reduction.sync(group)
+    for k, accs in zip(keys, want):
+        for r, acc in enumerate(reduction.get_peer_accumulations(k)):
+            assert_bit_equal(acc, accs[r], f"param {k} rank {r}")

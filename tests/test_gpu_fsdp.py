@@ -1,0 +1,114 @@
+"""FSDP glue on the GPU: the flat-parameter call sites and hooks (fsdp1) and the parameter-group
+layout with fused and two-step data flow (fsdp2), against the CPU oracle."""
+
+import math
+import types
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def test_fsdp1_hooks_and_call_sites(make_world):
+    """One minibatch the way examples/llm_training/torch_fsdp.py:462-481 drives it:
+    pre_minibatch_start, per microbatch gather + reduce_grad for two flat params, then
+    pre_optimizer_step publishes flat_param.grad = acc / factor in the parameter dtype."""
+    import odc_amd
+    from odc_amd.fsdp import fsdp1
+
+    W, M = 8, 3
+    group = make_world(W, 16 << 20)
+    fsdp1.patch_fsdp1(reduce_dtype=torch.float32)
+    g = torch.Generator().manual_seed(1)
+    numels = [100_003, 4096 * 8 + 5]
+    fulls = [(torch.randn(n, generator=g) * 0.02).bfloat16() for n in numels]
+    flat_params, handles = [], []
+    for full in fulls:
+        holder = torch.nn.Parameter(full.clone().cuda(), requires_grad=False)
+        for r in range(W):
+            sharded, pad = fsdp1.get_shard(holder, r, W)
+            assert_bit_equal(sharded, oracle.fsdp1_get_shard(full, r, W), f"shard {r}")
+        local = odc_amd.SymmBufferRegistry.get_instance().get_symm_buffer(id(holder))
+        holder.data = local  # FSDP points flat_param.data at the local shard
+        flat = types.SimpleNamespace(data=local, holder=holder)
+        flat_params.append(flat)
+        handles.append(types.SimpleNamespace(flat_param=holder))
+    module = types.SimpleNamespace(process_group=group, _gradient_postdivide_factor=float(W), _all_handles=handles)
+
+    fsdp1.pre_minibatch_start(module)
+    want = [[torch.zeros(math.ceil(n / W)) for _ in range(W)] for n in numels]
+    for _ in range(M):
+        for i, (flat, full) in enumerate(zip(flat_params, fulls)):
+            S = math.ceil(numels[i] / W)
+            out = torch.empty(W * S, dtype=torch.bfloat16, device="cuda")
+            fsdp1.all_gather_flat_param(out, flat.data, group)
+            assert_bit_equal(out[: numels[i]], full, "gathered flat param")
+            grad = (torch.randn(numels[i], generator=g) * 1e-3).bfloat16()
+            saved = fsdp1.reduce_grad(flat.holder, grad.cuda(), group)
+            assert saved.data_ptr() == fsdp1.get_reduction_service().get_accumulation(id(flat.holder)).data_ptr()
+            oracle.scatter_accumulate(want[i], oracle.fsdp1_pad_grad(grad, W))
+    fsdp1.pre_optimizer_step(module)
+    for i, handle in enumerate(handles):
+        expect = oracle.fsdp1_publish(want[i][0].clone(), float(W), torch.bfloat16)
+        assert handle.flat_param.grad.dtype == torch.bfloat16
+        assert_bit_equal(handle.flat_param.grad, expect, f"published grad {i}")
+    # the next minibatch starts from zero again
+    fsdp1.pre_minibatch_start(module)
+    fsdp1.get_reduction_service().sync(group)
+    for h in handles:
+        acc = fsdp1.get_reduction_service().get_accumulation(id(h.flat_param))
+        assert not acc.cpu().any()
+
+
+@pytest.mark.parametrize("W", [4, 8, 12])
+@pytest.mark.parametrize("fused", [True, False])
+def test_fsdp2_group_layout(make_world, W, fused):
+    """A parameter group with uneven dim 0 (padding rows, empty tail shards): unshard and reduce,
+    fused and two-step, equal the oracle built from torch._chunk_cat / split_with_sizes_copy."""
+    from odc_amd import virtual_rank
+    from odc_amd.fsdp import fsdp2
+
+    group = make_world(W, 32 << 20)
+    fsdp2.patch_fsdp2()
+    fsdp2.reduction_service.accumulation_dtype = None
+    shapes = [(37, 24), (5,), (64, 16), (3, 7, 2), (1024, 96), (W + 1, 33)]
+    g = torch.Generator().manual_seed(W)
+    params = [(torch.randn(*s, generator=g) * 0.02).bfloat16() for s in shapes]
+    pgp = fsdp2.ParamGroup(shapes, torch.bfloat16, group, reduce_dtype=torch.float32, name="blk")
+    pgp.load_full_params([p.cuda() for p in params])
+
+    packed = oracle.fsdp2_pack_shards(params, W)
+    from odc_amd import SymmBufferRegistry
+
+    for r, buf in enumerate(SymmBufferRegistry.get_instance().peer_tensors[pgp.key]):
+        assert_bit_equal(buf, packed[r], f"packed shard of rank {r}")
+    unsharded = pgp.unshard(fused=fused)
+    want = oracle.fsdp2_copy_out(oracle.gather(packed), shapes, W)
+    for p, (u, w, full) in enumerate(zip(unsharded, want, params)):
+        assert_bit_equal(u, w, f"unsharded param {p}")
+        assert_bit_equal(u, full, f"unsharded param {p} vs original")
+
+    module = types.SimpleNamespace(_odc_param_groups=[pgp])
+    fsdp2.pre_minibatch_start(module)
+    accs = [torch.zeros(pgp.total_shard_numel) for _ in range(W)]
+    for _ in range(3):
+        grads = [(torch.randn(*s, generator=g) * 1e-3).bfloat16() for s in shapes]
+        pgp.reduce([x.cuda() for x in grads], fused=fused)
+        oracle.scatter_accumulate(accs, oracle.fsdp2_copy_in(grads, W, torch.float32))
+    for r in range(W):
+        with virtual_rank(r):
+            if r == 0:
+                fsdp2.pre_optimizer_step(module)
+                got = pgp.sharded_grads
+            else:
+                pgp._reduced = True
+                got = pgp.update_gradients()
+            wantv = oracle.fsdp2_grad_views(oracle.fsdp2_average(accs[r].clone(), W).bfloat16(), shapes, W, r)
+            for p, (a, b) in enumerate(zip(got, wantv)):
+                assert tuple(a.shape) == tuple(b.shape), f"rank {r} param {p}"
+                assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
+    assert set(fsdp2.get_symm_buffer_memory_breakdown()) >= {"fsdp_params", "accumulation"}

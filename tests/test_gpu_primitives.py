@@ -12,21 +12,7 @@ from oracle import odc_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
-def bits(t: torch.Tensor) -> torch.Tensor:
-    """Integer view for bit-exact comparison (NaN-safe)."""
-    return t.contiguous().view({1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
-
-
-def assert_bit_equal(got: torch.Tensor, want: torch.Tensor, what=""):
-    got, want = got.cpu(), want.cpu()
-    assert got.shape == want.shape and got.dtype == want.dtype, what
-    if not torch.equal(bits(got), bits(want)):
-        bad = (bits(got) != bits(want)).nonzero().flatten()
-        i = int(bad[0])
-        raise AssertionError(
-            f"{what}: {bad.numel()} of {got.numel()} elements differ; first at {i}: "
-            f"got {got.flatten()[i].item()!r} want {want.flatten()[i].item()!r}"
-        )
+from helpers import assert_bit_equal, bits  # noqa: E402,F401
 
 
 def services():
@@ -36,17 +22,9 @@ def services():
 
 
 def put_shards(registry, key, shards, group):
-    """Each virtual rank publishes its shard, as each process does in the reference
-    (examples/all_gather.py:82-84)."""
-    from odc_amd import virtual_rank
+    from helpers import put_shards as _put
 
-    local = None
-    for r, s in enumerate(shards):
-        with virtual_rank(r):
-            t = registry.update_symm_buffer(key, s.cuda())
-            if r == 0:
-                local = t
-    return local
+    return _put(registry, key, shards)
 
 
 def test_gather_known_answer_pattern(make_world):
