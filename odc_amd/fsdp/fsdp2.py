@@ -193,7 +193,10 @@ class ParamGroup:
                 acc *= d
             stride = (acc, *reversed(inner))
             grads.append(
-                torch.as_strided(reduce_output, size=size, stride=stride, storage_offset=self.offsets[p])
+                torch.as_strided(
+                    reduce_output, size=size, stride=stride,
+                    storage_offset=reduce_output.storage_offset() + self.offsets[p],
+                )
             )
         self.sharded_grads = grads
         return grads

@@ -163,8 +163,13 @@ class SymmetricArena:
         nbytes = numel * dtype.itemsize
         if not 0 <= rank < self.world_size or offset + nbytes > self.bytes_per_rank:
             raise ValueError(f"view of rank {rank} [{offset}, +{nbytes}) leaves the rank region")
-        start = rank * self.rank_stride + offset
-        return self._bytes[start : start + nbytes].view(dtype).view(tuple(shape))
+        if nbytes == 0:
+            return torch.empty(tuple(shape), dtype=dtype, device=self._bytes.device)
+        # a tensor of its own (storage offset 0), so that callers may as_strided into it with
+        # absolute offsets the way odc/fsdp/fsdp2.py:902-907 does
+        mem = _ArenaMemory(self.base + rank * self.rank_stride + offset, nbytes)
+        flat = torch.as_tensor(mem, device=self._bytes.device)
+        return flat.view(dtype).view(tuple(shape))
 
     def destroy(self) -> None:
         if self._handle is not None and self._handle.value:

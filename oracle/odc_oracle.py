@@ -214,13 +214,10 @@ def fsdp2_grad_views(
         chunk_rows = math.ceil(s[0] / world_size)
         rows = max(0, min(chunk_rows, s[0] - rank * chunk_rows))
         size = (rows, *s[1:])
-        stride = []
-        acc_stride = 1
-        for d in reversed(size[1:] if len(size) > 1 else ()):
-            stride.append(acc_stride)
-            acc_stride *= d
-        stride = (acc_stride, *reversed(stride)) if len(size) >= 1 else ()
-        views.append(torch.as_strided(acc, size=size, stride=stride, storage_offset=offset))
+        stride = torch.empty(max(rows, 1), *s[1:]).stride()  # contiguous strides of the shard
+        views.append(
+            torch.as_strided(acc, size=size, stride=stride, storage_offset=acc.storage_offset() + offset)
+        )
         offset += fsdp2_padded_shard_numel(s, world_size)
     return views
 

@@ -66,7 +66,8 @@ def test_fsdp1_hooks_and_call_sites(make_world):
 
 @pytest.mark.parametrize("W", [4, 8, 12])
 @pytest.mark.parametrize("fused", [True, False])
-def test_fsdp2_group_layout(make_world, W, fused):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fsdp2_group_layout(make_world, W, fused, dtype):
     """A parameter group with uneven dim 0 (padding rows, empty tail shards): unshard and reduce,
     fused and two-step, equal the oracle built from torch._chunk_cat / split_with_sizes_copy."""
     from odc_amd import virtual_rank
@@ -77,8 +78,8 @@ def test_fsdp2_group_layout(make_world, W, fused):
     fsdp2.reduction_service.accumulation_dtype = None
     shapes = [(37, 24), (5,), (64, 16), (3, 7, 2), (1024, 96), (W + 1, 33)]
     g = torch.Generator().manual_seed(W)
-    params = [(torch.randn(*s, generator=g) * 0.02).bfloat16() for s in shapes]
-    pgp = fsdp2.ParamGroup(shapes, torch.bfloat16, group, reduce_dtype=torch.float32, name="blk")
+    params = [(torch.randn(*s, generator=g) * 0.02).to(dtype) for s in shapes]
+    pgp = fsdp2.ParamGroup(shapes, dtype, group, reduce_dtype=torch.float32, name="blk")
     pgp.load_full_params([p.cuda() for p in params])
 
     packed = oracle.fsdp2_pack_shards(params, W)
@@ -96,7 +97,7 @@ def test_fsdp2_group_layout(make_world, W, fused):
     fsdp2.pre_minibatch_start(module)
     accs = [torch.zeros(pgp.total_shard_numel) for _ in range(W)]
     for _ in range(3):
-        grads = [(torch.randn(*s, generator=g) * 1e-3).bfloat16() for s in shapes]
+        grads = [(torch.randn(*s, generator=g) * 1e-3).to(dtype) for s in shapes]
         pgp.reduce([x.cuda() for x in grads], fused=fused)
         oracle.scatter_accumulate(accs, oracle.fsdp2_copy_in(grads, W, torch.float32))
     for r in range(W):
@@ -107,8 +108,13 @@ def test_fsdp2_group_layout(make_world, W, fused):
             else:
                 pgp._reduced = True
                 got = pgp.update_gradients()
-            wantv = oracle.fsdp2_grad_views(oracle.fsdp2_average(accs[r].clone(), W).bfloat16(), shapes, W, r)
+            wantv = oracle.fsdp2_grad_views(oracle.fsdp2_average(accs[r].clone(), W).to(dtype), shapes, W, r)
             for p, (a, b) in enumerate(zip(got, wantv)):
                 assert tuple(a.shape) == tuple(b.shape), f"rank {r} param {p}"
-                assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
+                if W & (W - 1) == 0:
+                    assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
+                else:
+                    # the averaging is torch's own `/=` on the device, which multiplies by the
+                    # rounded reciprocal of a scalar divisor: exact only for powers of two
+                    torch.testing.assert_close(a.cpu(), b, rtol=1e-6, atol=0)
     assert set(fsdp2.get_symm_buffer_memory_breakdown()) >= {"fsdp_params", "accumulation"}

@@ -1,0 +1,234 @@
+"""Host-side logic that needs no GPU: the C ABI surface, the arena's offset bookkeeping (on an
+arena without device memory), the registry and splitter mirrors, error behaviour, and the rule
+that the product never reaches for the oracle or a CPU fallback."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from odc_amd import _native
+from odc_amd.primitives import utils
+from oracle import odc_oracle as oracle
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+# ---- C ABI -------------------------------------------------------------------------------------
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "odc_hip.h").read_text()
+    declared = set(re.findall(r"\b(odc_[a-z_]+)\s*\(", header))
+    assert declared == set(_native.EXPORTED_SYMBOLS)
+    lib = _native.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/odc_hip.h but not exported"
+    assert lib.odc_abi_version() == _native.ABI_VERSION == int(re.search(r"ODC_HIP_ABI_VERSION (\d+)", header).group(1))
+    assert _native.MAX_ITEMS_PER_LAUNCH == int(re.search(r"ODC_MAX_ITEMS_PER_LAUNCH (\d+)", header).group(1))
+
+
+def test_struct_layouts_match_the_header():
+    assert ctypes.sizeof(_native.GatherItem) == 24
+    assert ctypes.sizeof(_native.AccumItem) == 32
+    assert ctypes.sizeof(_native.Span) == 16
+    assert ctypes.sizeof(_native.ArenaInfo) == 4 * 4 + 5 * 8
+
+
+def test_options_roundtrip_and_unknown_name():
+    old = _native.get_option("gather_blocks_per_cu")
+    _native.set_option("gather_blocks_per_cu", 3)
+    assert _native.get_option("gather_blocks_per_cu") == 3
+    _native.set_option("gather_blocks_per_cu", old)
+    with pytest.raises(_native.OdcNativeError) as e:
+        _native.set_option("no_such_knob", 1)
+    assert e.value.code == _native.ODC_ERR_INVALID and "no_such_knob" in e.value.message
+    with pytest.raises(_native.OdcNativeError):
+        _native.set_option("rank_major", -1)
+
+
+# ---- arena bookkeeping (no device memory) ------------------------------------------------------
+def test_arena_offsets_first_fit_and_coalescing():
+    a = utils.SymmetricArena(8, 1 << 20, backing=False)
+    info = a.info()
+    assert (info.world_size, info.device, info.base, info.bytes_per_rank) == (8, -1, 0, 1 << 20)
+    assert info.rank_stride >= info.bytes_per_rank
+    o = [a.alloc(n) for n in (100, 1000, 1, 0, 4096)]
+    assert o == [0, 256, 1280, 1536, 1792]  # 256 B granules, bump order
+    assert a.info().bytes_in_use == 256 + 1024 + 256 + 256 + 4096 and a.info().n_allocations == 5
+    a.free(o[1])
+    a.free(o[2])  # merges with the freed block before it
+    assert a.alloc(1280) == 256  # fits exactly into the merged hole
+    a.free(o[0])
+    assert a.alloc(10) == 0
+    with pytest.raises(_native.OdcNativeError) as e:
+        a.free(12345)
+    assert e.value.code == _native.ODC_ERR_NOT_FOUND
+    hw = a.info().high_water
+    a.reset()
+    assert a.info().bytes_in_use == 0 and a.info().n_allocations == 0 and a.info().high_water == hw
+    assert a.alloc(1 << 20) == 0
+    with pytest.raises(_native.OdcNativeError) as e:
+        a.alloc(1)
+    assert e.value.code == _native.ODC_ERR_NOMEM
+    a.destroy()
+    with pytest.raises(RuntimeError):
+        a.alloc(1)  # use after finalize
+
+
+def test_sizing_run_for_the_8b_layer():
+    """What the bookkeeping-only arena is for: learn the bytes per rank a workload needs."""
+    from odc_amd.workloads import llama3_8b_layer_shapes, numel
+
+    W = 8
+    a = utils.SymmetricArena(W, 1 << 40, backing=False)
+    for _, shape in llama3_8b_layer_shapes():
+        a.alloc(numel(shape) // W * 2)  # bf16 shard
+        a.alloc(numel(shape) // W * 4)  # fp32 accumulation
+    need = a.info().high_water
+    assert 27_264_000 * 6 <= need <= 27_264_000 * 6 + 18 * 256
+    a.destroy()
+
+
+def test_bad_arguments_and_compute_on_unbacked_arena():
+    lib = _native.load()
+    h = ctypes.c_void_p()
+    assert lib.odc_arena_create(0, 1024, 0, ctypes.byref(h)) == _native.ODC_ERR_INVALID
+    assert lib.odc_arena_create(4, 0, 0, ctypes.byref(h)) == _native.ODC_ERR_INVALID
+    assert lib.odc_arena_create(4, 1024, 0x80, ctypes.byref(h)) == _native.ODC_ERR_INVALID
+    assert lib.odc_arena_create(4, 1024, 0, None) == _native.ODC_ERR_INVALID
+    assert lib.odc_arena_destroy(None) == _native.ODC_ERR_INVALID
+    a = utils.SymmetricArena(4, 1 << 16, backing=False)
+    items = (_native.GatherItem * 1)()
+    assert lib.odc_gather(a.handle, items, 1, 0, None) == _native.ODC_ERR_NO_BACKING
+    acc = (_native.AccumItem * 1)()
+    assert lib.odc_scatter_accumulate(a.handle, acc, 1, 0, 2, None) == _native.ODC_ERR_NO_BACKING
+    spans = (_native.Span * 1)()
+    assert lib.odc_clear(a.handle, spans, 1, None) == _native.ODC_ERR_NO_BACKING
+    assert b"no device memory" in lib.odc_last_error()
+    assert lib.odc_arena_ptr(a.handle, 0, 0) is None
+    assert lib.odc_arena_locate(a.handle, ctypes.c_void_p(64), None, None, None) == _native.ODC_ERR_NO_BACKING
+    with pytest.raises(RuntimeError):
+        a.view(0, 0, (4,), torch.float32)
+    a.destroy()
+
+
+def test_product_fails_loudly_without_a_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("this check is for the CPU-only container")
+    with pytest.raises(RuntimeError):
+        utils.init_nvshmem(world_size=4, symmetric_size="1M")
+    with pytest.raises(_native.OdcNativeError) as e:
+        utils.SymmetricArena(4, 1 << 20)  # hipMalloc has no device to run on
+    assert e.value.code == _native.ODC_ERR_HIP
+    with pytest.raises(RuntimeError):
+        utils.get_rank()  # no world
+
+
+def test_product_never_imports_the_oracle():
+    for path in (ROOT / "odc_amd").rglob("*"):
+        if path.suffix in (".py", ".hip", ".h", ".cpp"):
+            text = path.read_text()
+            assert "oracle" not in text.lower(), f"{path} mentions the oracle"
+    assert "oracle" not in (ROOT / "include" / "odc_hip.h").read_text().lower()
+
+
+# ---- mirrors of the reference's host classes ---------------------------------------------------
+@pytest.mark.parametrize("env,shape,W", [
+    (None, (27_264_000,), 8), (None, (7_340_032,), 8), (None, (512,), 8), (None, (100,), 8),
+    ("0", (100,), 8), ("-1", (1000, 3), 12), ("1024", (1000, 3), 4), (None, (218_112_000,), 8),
+    ("4096", (10,), 64),
+])
+def test_buffer_splitter_matches_the_oracle(monkeypatch, env, shape, W):
+    if env is None:
+        monkeypatch.delenv("ODC_MAX_BUFFER_SIZE", raising=False)
+    else:
+        monkeypatch.setenv("ODC_MAX_BUFFER_SIZE", env)
+    mine, ref = utils.BufferSplitter(), oracle.BufferSplitter()
+    assert mine.get_global_buffer_size(shape) == ref.get_global_buffer_size(shape)
+    assert mine.get_local_buffer_size(shape, W) == ref.get_local_buffer_size(shape, W)
+
+
+def test_buffer_splitter_assertion(monkeypatch):
+    monkeypatch.delenv("ODC_MAX_BUFFER_SIZE", raising=False)
+    with pytest.raises(AssertionError, match="ODC_MAX_BUFFER_SIZE"):
+        utils.BufferSplitter().get_local_buffer_size((100,), 12)
+
+
+def test_parse_size():
+    assert utils.parse_size("30G") == 30 * 2**30
+    assert utils.parse_size("5000000000") == 5_000_000_000
+    assert utils.parse_size("512m") == 512 * 2**20
+    assert utils.parse_size("1.5GB") == int(1.5 * 2**30)
+    assert utils.parse_size(4096) == 4096
+
+
+class _HostArena:
+    """Stand-in arena over host memory, for the registry's bookkeeping only."""
+
+    def __init__(self, world_size, nbytes):
+        self.world_size = world_size
+        self.mem = [torch.zeros(nbytes, dtype=torch.uint8) for _ in range(world_size)]
+        self.top = 0
+        self.freed = []
+
+    def alloc(self, nbytes):
+        off = self.top
+        self.top += max(256, -(-nbytes // 256) * 256)
+        return off
+
+    def free(self, offset):
+        self.freed.append(offset)
+
+    def view(self, rank, offset, shape, dtype):
+        n = torch.Size(shape).numel() * dtype.itemsize
+        return self.mem[rank][offset : offset + n].view(dtype).view(shape)
+
+
+def test_registry_bookkeeping_on_a_host_arena():
+    current = {"rank": 0}
+    reg = utils.SymmBufferRegistry(arena=_HostArena(3, 1 << 16), rank_fn=lambda: current["rank"])
+    t = reg.allocate_symm_buffer("w", (10,), torch.float32)
+    assert reg.has_key("w") and not reg.has_key("x") and reg.is_nvshmem_tensor(t)
+    with pytest.raises(AssertionError):
+        reg.allocate_symm_buffer("w", (10,), torch.float32)  # utils.py:127
+    with pytest.raises(ValueError, match="not found"):
+        reg.get_symm_buffer("x")  # utils.py:153-156
+    assert reg.get_or_create_symm_buffer("w", (10,), torch.float32).data_ptr() == t.data_ptr()
+    peers = reg.get_peer_tensors(t)
+    assert len(peers) == 3 and len({p.data_ptr() for p in peers}) == 3
+    # update copies once per rank until flush (utils.py:103-116)
+    assert torch.equal(reg.update_symm_buffer("w", torch.arange(10.0)), torch.arange(10.0))
+    assert torch.equal(reg.update_symm_buffer("w", torch.zeros(10)), torch.arange(10.0))
+    current["rank"] = 2
+    assert torch.equal(reg.update_symm_buffer("w", torch.ones(10)), torch.ones(10))  # rank 2's first
+    assert torch.equal(peers[0], torch.arange(10.0)) and not peers[1].any()
+    assert reg.get_symm_buffer("w").data_ptr() == peers[2].data_ptr()
+    assert reg.local_tensor["w"].data_ptr() == peers[2].data_ptr()
+    reg.flush()
+    assert torch.equal(reg.update_symm_buffer("w", torch.full((10,), 7.0)), torch.full((10,), 7.0))
+    reg.update_symm_buffer(("k", 1), torch.zeros(4, dtype=torch.bfloat16))  # lazily allocates
+    assert reg.memory_allocated() == 40 + 8
+    reg.finalize()
+    assert sorted(reg._arena.freed) == [0, 256] and not reg.has_key("w") and reg.memory_allocated() == 0
+
+
+def test_services_refuse_host_tensors():
+    from odc_amd import GatherService, ReductionService
+
+    if utils.is_initialized():
+        pytest.skip("a world exists")
+    with pytest.raises(RuntimeError):  # no arena, no compute
+        GatherService().gather_into_tensor(torch.empty(8), torch.empty(2), utils.VirtualGroup(4))
+    with pytest.raises(RuntimeError):
+        ReductionService().scatter_accumulate("k", torch.empty(8), utils.VirtualGroup(4))
+
+
+def test_workload_shapes():
+    from odc_amd import workloads as w
+
+    assert sum(w.numel(s) for _, s in w.llama3_8b_layer_shapes()) == 218_112_000
+    assert sum(w.numel(s) for _, unit in w.llama3_8b_units() for _, s in unit) == 8_030_261_248
+    sizes = w.uneven_flat_numels()
+    assert len(sizes) == 40 and all(4096 <= n <= 58_720_256 + 12 and n % 12 for n in sizes)
+    assert sizes == w.uneven_flat_numels()  # deterministic
