@@ -8,7 +8,8 @@ One step = one microbatch of the path over the whole layer:
 Every 8th step starts a new minibatch and first clears the accumulations (inside the timed
 region; its 4N written bytes are NOT counted in the numerator).
 
-Prints ONE JSON line (see README / DESIGN for the fields).
+Prints ONE JSON line: whole-step throughput, per-kernel roofline figures from HIP events on the
+launch stream, the CPU oracle timed on the host cores, and the parity verdict.
 """
 
 from __future__ import annotations
