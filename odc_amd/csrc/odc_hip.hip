@@ -434,14 +434,40 @@ int check_arena(const odc_arena* a) {
   return ODC_OK;
 }
 
-int check_compute(odc_arena* a) {
+// Makes the arena's device current for the scope of one entry point and puts the caller's
+// device back afterwards (the caller may be any host thread with any current device).
+class DeviceGuard {
+ public:
+  DeviceGuard() = default;
+  DeviceGuard(const DeviceGuard&) = delete;
+  DeviceGuard& operator=(const DeviceGuard&) = delete;
+  int enter(int device) {
+    ODC_HIP_TRY(hipGetDevice(&prev_));
+    if (prev_ != device) {
+      ODC_HIP_TRY(hipSetDevice(device));
+      switched_ = true;
+    }
+    return ODC_OK;
+  }
+  ~DeviceGuard() {
+    if (switched_) (void)hipSetDevice(prev_);
+  }
+
+ private:
+  int prev_ = -1;
+  bool switched_ = false;
+};
+
+int check_compute(odc_arena* a, DeviceGuard& guard) {
   if (int rc = check_arena(a)) return rc;
   if (!a->base)
     return fail(ODC_ERR_NO_BACKING, "arena has no device memory (created with ODC_ARENA_NO_BACKING)");
-  int cur = -1;
-  ODC_HIP_TRY(hipGetDevice(&cur));
-  if (cur != a->device) ODC_HIP_TRY(hipSetDevice(a->device));
-  return ODC_OK;
+  return guard.enter(a->device);
+}
+
+Options options_snapshot() {
+  std::lock_guard<std::mutex> lk(g_opt_mu);
+  return g_opt;
 }
 
 uint32_t grid_for(const odc_arena* a, int64_t blocks_per_cu, uint32_t n_tiles) {
@@ -489,7 +515,7 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
   a->world = world_size;
   a->flags = flags;
   a->bytes_per_rank = round_up(bytes_per_rank, kAlign);
-  a->rank_stride = a->bytes_per_rank + round_up((uint64_t)g_opt.rank_stagger_bytes, kAlign);
+  a->rank_stride = a->bytes_per_rank + round_up((uint64_t)options_snapshot().rank_stagger_bytes, kAlign);
   if (a->rank_stride > (~0ull) / world_size) {
     delete a;
     return fail(ODC_ERR_INVALID, "arena size overflows 64 bits");
@@ -641,7 +667,8 @@ int odc_arena_locate(const odc_arena* a, const void* ptr, uint32_t* rank, uint64
 // ------------------------------------------------------------------------------------------------
 int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uint32_t first_rank,
                void* stream) {
-  if (int rc = check_compute(a)) return rc;
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
   if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
   if (first_rank >= a->world)
     return fail(ODC_ERR_INVALID, "first_rank %u >= world size %u", first_rank, a->world);
@@ -666,7 +693,7 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
       }
     }
   }
-  const Options opt = g_opt;
+  const Options opt = options_snapshot();
   uint32_t i = 0;
   while (i < n_items) {
     GatherLaunch L;
@@ -704,7 +731,8 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
 }
 
 int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* stream) {
-  if (int rc = check_compute(a)) return rc;
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
   if (n_spans && !spans) return fail(ODC_ERR_INVALID, "spans is NULL");
   for (uint32_t i = 0; i < n_spans; ++i) {
     if (spans[i].offset > a->bytes_per_rank || spans[i].nbytes > a->bytes_per_rank - spans[i].offset)
@@ -712,7 +740,7 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
                   (unsigned long long)spans[i].offset, (unsigned long long)spans[i].nbytes,
                   (unsigned long long)a->bytes_per_rank);
   }
-  const Options opt = g_opt;
+  const Options opt = options_snapshot();
   uint32_t i = 0;
   while (i < n_spans) {
     ClearLaunch L;
@@ -779,7 +807,8 @@ accum_fn pick_accum(int g, int a) {
 
 extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
                                       int grad_dtype, int acc_dtype, void* stream) {
-  if (int rc = check_compute(a)) return rc;
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
   if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
   const int gb = dtype_bytes(grad_dtype), ab = dtype_bytes(acc_dtype);
   if (!gb || !ab) return fail(ODC_ERR_INVALID, "unknown dtype code (grad %d, acc %d)", grad_dtype, acc_dtype);
@@ -810,7 +839,7 @@ extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items,
     if ((uintptr_t)it.grad % gb)
       return fail(ODC_ERR_INVALID, "item %u: grad pointer is not aligned to the gradient dtype", i);
   }
-  const Options opt = g_opt;
+  const Options opt = options_snapshot();
   uint32_t i = 0;
   while (i < n_items) {
     AccumLaunch L;

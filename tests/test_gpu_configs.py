@@ -116,3 +116,69 @@ def test_config3_uneven_padded_w12(make_world):
     for k, accs in zip(keys, want):
         for r, acc in enumerate(reduction.get_peer_accumulations(k)):
             assert_bit_equal(acc, accs[r], f"param {k} rank {r}")
+
+
+def test_config5_full_llama3_8b_sweep(make_world):
+    """Full Llama-3-8B (34 FSDP units: embedding, 32 layers, final norm + untied lm_head; 8.03 G
+    bf16 parameters, W=8, ~48 GB arena). Per microbatch: gather unit by unit in forward order, then
+    scatter-accumulate unit by unit in reverse order. Values come from per-(unit, microbatch) seeded
+    device generators, so they can be drawn again for checking:
+      * every unit: gathered parameters equal the regenerated parameters; accumulations equal
+        (0 + g0) + g1 computed with torch's fp32 add on the device (an independent implementation);
+      * sampled units (embedding, two layers, head): bit-exact against the CPU oracle."""
+    from odc_amd import virtual_rank
+    from odc_amd.workloads import llama3_8b_units
+
+    W, M = 8, 2
+    units = llama3_8b_units()
+    total = sum(numel(s) for _, unit in units for _, s in unit)
+    assert total == 8_030_261_248
+    per_rank = sum((numel(s) // W) * 6 + 512 for _, unit in units for _, s in unit) + (1 << 20)
+    group = make_world(W, per_rank)
+    gather, reduction, registry = _services()
+
+    def draw(u, p, m, n, scale):
+        gen = torch.Generator(device="cuda").manual_seed(1_000_003 * u + 1009 * p + m)
+        return device_randn_bf16(n, gen, scale)
+
+    keys = []
+    for u, (_, unit) in enumerate(units):
+        ks = []
+        for p, (_, shape) in enumerate(unit):
+            n = numel(shape)
+            full = draw(u, p, -1, n, 0.02)
+            for r in range(W):
+                with virtual_rank(r):
+                    registry.update_symm_buffer((u, p), full.view(W, -1)[r])
+            reduction.register((u, p), (n // W,), torch.bfloat16, torch.float32, group)
+            ks.append((u, p))
+        keys.append(ks)
+    sampled = {0, 1, 17, len(units) - 1}
+    outs_by_shape = {}
+    for m in range(M):
+        for u, (_, unit) in enumerate(units):  # forward: gather
+            sig = tuple(numel(s) for _, s in unit)
+            if sig not in outs_by_shape:
+                outs_by_shape[sig] = [torch.empty(n, dtype=torch.bfloat16, device="cuda") for n in sig]
+            outs = outs_by_shape[sig]
+            gather.gather_into_tensors(outs, [registry.get_symm_buffer(k) for k in keys[u]], group)
+            if m == 0:
+                for p, o in enumerate(outs):
+                    assert torch.equal(o.view(torch.int16), draw(u, p, -1, o.numel(), 0.02).view(torch.int16)), (u, p)
+        for u in reversed(range(len(units))):  # backward: scatter-accumulate
+            grads = [draw(u, p, m, numel(s), 1e-3) for p, (_, s) in enumerate(units[u][1])]
+            reduction.scatter_accumulate_multi(keys[u], grads, group)
+    reduction.sync(group)
+    for u, (_, unit) in enumerate(units):
+        for p, (_, shape) in enumerate(unit):
+            n = numel(shape)
+            g0, g1 = draw(u, p, 0, n, 1e-3), draw(u, p, 1, n, 1e-3)
+            expect = (torch.zeros(n, device="cuda") + g0.float()) + g1.float()
+            got = torch.cat(list(reduction.get_peer_accumulations((u, p))))
+            assert torch.equal(got.view(torch.int32), expect.view(torch.int32)), (u, p)
+            if u in sampled:
+                accs = [torch.zeros(n // W) for _ in range(W)]
+                oracle.scatter_accumulate(accs, g0.cpu())
+                oracle.scatter_accumulate(accs, g1.cpu())
+                assert_bit_equal(got, torch.cat(accs), f"unit {u} param {p} vs oracle")
+            del g0, g1, expect, got

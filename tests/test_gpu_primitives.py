@@ -156,3 +156,46 @@ def test_scatter_accumulate_special_values(make_world):
     for r, acc in enumerate(reduction.get_peer_accumulations("d")):
         assert_bit_equal(acc, wantd[r], "denormal")
         assert (acc.cpu() != 0).all()
+
+
+def test_hip_graph_capture_and_replay(make_world):
+    """No entry point allocates, synchronises or memsets, so clear + scatter-accumulate + gather
+    can be captured in a HIP graph; every replay (with eager work and synchronisations between
+    replays) must reproduce the eager result."""
+    from odc_amd import virtual_rank
+
+    W, S = 8, 50_003
+    group = make_world(W, 16 << 20)
+    gather, reduction, registry = services()
+    g = torch.Generator().manual_seed(9)
+    shards = [(torch.randn(S, generator=g) * 0.02).bfloat16() for _ in range(W)]
+    src = put_shards(registry, "p", shards, group)
+    grad = (torch.randn(W * S, generator=g) * 1e-3).bfloat16().cuda()
+    grad2 = (torch.randn(W * S, generator=g) * 1e-3).bfloat16()
+    out = torch.zeros(W * S, dtype=torch.bfloat16, device="cuda")
+    reduction.register("p", (S,), torch.bfloat16, torch.float32, group)
+    reduction.sync(group)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        reduction.clear_accumulations()
+        reduction.scatter_accumulate("p", grad, group)
+        reduction.scatter_accumulate("p", grad, group)
+        gather.gather_into_tensor(out, src, group)
+    want_acc = [torch.zeros(S) for _ in range(W)]
+    oracle.scatter_accumulate(want_acc, grad.cpu())
+    oracle.scatter_accumulate(want_acc, grad.cpu())
+    for replay in range(4):
+        # eager work between replays: dirty the outputs, move the inputs' values
+        out.fill_(7.0)
+        reduction.scatter_accumulate("p", grad2.cuda(), group)
+        with virtual_rank(replay % W):
+            registry.get_symm_buffer("p").add_(1.0)
+        shards[replay % W] = (shards[replay % W].float() + 1.0).bfloat16()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bit_equal(out, oracle.gather(shards), f"replay {replay}: gather")
+        for r, acc in enumerate(reduction.get_peer_accumulations("p")):
+            assert_bit_equal(acc, want_acc[r], f"replay {replay}: accumulation of rank {r}")
