@@ -122,6 +122,22 @@ int odc_gather(odc_arena* arena, const odc_gather_item* items, uint32_t n_items,
                uint32_t first_rank, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * gather with cast — the same as gather, but shards of src_dtype are converted to dst_dtype on
+ * the way (exact widening, round-to-nearest-even narrowing):
+ *     dst[r*shard_elems + i] = cast(rank r's element i at src_offset)
+ * One pass instead of the reference's gather in the shard dtype followed by a cast of the full
+ * parameter (odc/fsdp/fsdp1.py:199-223, odc/fsdp/fsdp2.py:341-343).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct odc_gather_cast_item {
+  void* dst;             /* device pointer to W*shard_elems elements of dst_dtype */
+  uint64_t src_offset;   /* symmetric byte offset of the shard, src_dtype aligned */
+  uint64_t shard_elems;  /* elements contributed by each rank */
+} odc_gather_cast_item;
+
+int odc_gather_cast(odc_arena* arena, const odc_gather_cast_item* items, uint32_t n_items,
+                    int src_dtype, int dst_dtype, uint32_t first_rank, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * scatter-accumulate — for every item and every rank r, with g = the item's gradient viewed as
  * W consecutive chunks of shard_elems elements (elements at index >= grad_elems read as +0):
  *     acc_r[0:shard_elems] += g[r*shard_elems : (r+1)*shard_elems]
@@ -152,6 +168,22 @@ typedef struct odc_span {
 } odc_span;
 
 int odc_clear(odc_arena* arena, const odc_span* spans, uint32_t n_spans, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * publish — end-of-minibatch pass over ONE rank's accumulations, for every item:
+ *     acc[i] = acc[i] / divisor        (in place, correctly rounded; skipped when divisor == 1)
+ *     out[i] = cast_to_out_dtype(acc[i])                      (skipped when out is NULL)
+ * Replaces `acc /= W` / `_div_if_needed(acc, factor)` followed by `acc.to(param_dtype)`
+ * (odc/fsdp/fsdp1.py:324-335, odc/fsdp/fsdp2.py:846-847,897-899) with one read of the shard.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct odc_publish_item {
+  uint64_t acc_offset;   /* symmetric byte offset of the accumulation (slice), acc_dtype aligned */
+  uint64_t elems;
+  void* out;             /* device pointer to elems elements of out_dtype, or NULL */
+} odc_publish_item;
+
+int odc_publish(odc_arena* arena, uint32_t rank, const odc_publish_item* items, uint32_t n_items,
+                int acc_dtype, int out_dtype, float divisor, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Library-wide

@@ -30,8 +30,10 @@ EXPORTED_SYMBOLS = (
     "odc_arena_ptr",
     "odc_arena_locate",
     "odc_gather",
+    "odc_gather_cast",
     "odc_scatter_accumulate",
     "odc_clear",
+    "odc_publish",
     "odc_last_error",
     "odc_abi_version",
     "odc_set_option",
@@ -97,6 +99,22 @@ class AccumItem(ctypes.Structure):
     ]
 
 
+class GatherCastItem(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("src_offset", ctypes.c_uint64),
+        ("shard_elems", ctypes.c_uint64),
+    ]
+
+
+class PublishItem(ctypes.Structure):
+    _fields_ = [
+        ("acc_offset", ctypes.c_uint64),
+        ("elems", ctypes.c_uint64),
+        ("out", ctypes.c_void_p),
+    ]
+
+
 class Span(ctypes.Structure):
     _fields_ = [("offset", ctypes.c_uint64), ("nbytes", ctypes.c_uint64)]
 
@@ -158,7 +176,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.odc_arena_ptr.restype = vp
     lib.odc_arena_locate.argtypes = [vp, vp, P(u32), P(u64), P(u64)]
     lib.odc_gather.argtypes = [vp, P(GatherItem), u32, u32, vp]
+    lib.odc_gather_cast.argtypes = [vp, P(GatherCastItem), u32, ci, ci, u32, vp]
     lib.odc_scatter_accumulate.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
+    lib.odc_publish.argtypes = [vp, u32, P(PublishItem), u32, ci, ci, ctypes.c_float, vp]
     lib.odc_clear.argtypes = [vp, P(Span), u32, vp]
     lib.odc_last_error.argtypes = []
     lib.odc_last_error.restype = ctypes.c_char_p
@@ -182,7 +202,10 @@ def load() -> ctypes.CDLL:
                     "g.build()'` (needs hipcc). There is no fallback path."
                 )
             lib = ctypes.CDLL(str(LIB_PATH))
-            _declare(lib)
+            try:
+                _declare(lib)
+            except AttributeError as e:
+                raise ImportError(f"{LIB_PATH} is stale ({e}): rebuild it") from None
             got = lib.odc_abi_version()
             if got != ABI_VERSION:
                 raise ImportError(f"{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}: rebuild it")

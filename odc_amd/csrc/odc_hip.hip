@@ -91,31 +91,41 @@ constexpr uint32_t kTileElems = kTileVecs * 4;          // accumulate: 4096 elem
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Per-launch descriptors, passed by value (kernel argument segment, scalar loads).
-struct GatherLaunch {
-  const uint8_t* base;   // arena base (rank 0 region)
-  uint64_t rank_stride;
+// Per-launch descriptors, passed by value (kernel argument segment, scalar loads). Every launch
+// carries a TileTable: item i owns tiles [tile_prefix[i], tile_prefix[i+1]), which are
+// world * tiles_per_seg[i] tiles, one run of tiles_per_seg[i] per rank segment.
+struct TileTable {
   uint32_t world;
-  uint32_t first_rank;
   uint32_t n_items;
   uint32_t n_tiles;
   uint32_t rank_major;
+  uint32_t first_rank;
   uint32_t tile_prefix[kMaxItems + 1];
   uint32_t tiles_per_seg[kMaxItems];
+};
+
+struct GatherLaunch {
+  TileTable tt;
+  const uint8_t* base;   // arena base (rank 0 region)
+  uint64_t rank_stride;
   uint8_t* dst[kMaxItems];
   uint64_t src_off[kMaxItems];
   uint64_t seg_bytes[kMaxItems];
 };
 
+struct CastGatherLaunch {
+  TileTable tt;
+  const uint8_t* base;
+  uint64_t rank_stride;
+  uint8_t* dst[kMaxItems];
+  uint64_t src_off[kMaxItems];
+  uint64_t seg_elems[kMaxItems];
+};
+
 struct AccumLaunch {
+  TileTable tt;
   uint8_t* base;
   uint64_t rank_stride;
-  uint32_t world;
-  uint32_t n_items;
-  uint32_t n_tiles;
-  uint32_t rank_major;
-  uint32_t tile_prefix[kMaxItems + 1];
-  uint32_t tiles_per_seg[kMaxItems];
   const uint8_t* grad[kMaxItems];
   uint64_t grad_elems[kMaxItems];
   uint64_t acc_off[kMaxItems];
@@ -123,16 +133,21 @@ struct AccumLaunch {
 };
 
 struct ClearLaunch {
+  TileTable tt;
   uint8_t* base;
   uint64_t rank_stride;
-  uint32_t world;
-  uint32_t n_items;
-  uint32_t n_tiles;
-  uint32_t rank_major;
-  uint32_t tile_prefix[kMaxItems + 1];
-  uint32_t tiles_per_seg[kMaxItems];
   uint64_t off[kMaxItems];
   uint64_t seg_bytes[kMaxItems];
+};
+
+struct PublishLaunch {  // one rank's region only: tt.world == 1
+  TileTable tt;
+  uint8_t* region;      // base of the publishing rank's region
+  float divisor;
+  uint32_t divide;      // 0: leave the accumulation untouched
+  uint8_t* out[kMaxItems];  // may be null: divide in place only
+  uint64_t acc_off[kMaxItems];
+  uint64_t seg_elems[kMaxItems];
 };
 
 // Tile t of a launch -> (item, rank, chunk-in-segment). Everything here is wave-uniform.
@@ -140,26 +155,25 @@ struct TileCoord {
   uint32_t item, rank, chunk;
 };
 
-template <class L>
-__device__ __forceinline__ TileCoord locate_tile(const L& launch, uint32_t t, uint32_t first_rank) {
-  uint32_t lo = 0, hi = launch.n_items;  // largest i with tile_prefix[i] <= t
+__device__ __forceinline__ TileCoord locate_tile(const TileTable& tt, uint32_t t) {
+  uint32_t lo = 0, hi = tt.n_items;  // largest i with tile_prefix[i] <= t
   while (hi - lo > 1) {
     const uint32_t mid = (lo + hi) >> 1;
-    if (launch.tile_prefix[mid] <= t) lo = mid; else hi = mid;
+    if (tt.tile_prefix[mid] <= t) lo = mid; else hi = mid;
   }
-  const uint32_t lt = t - launch.tile_prefix[lo];
-  const uint32_t tps = launch.tiles_per_seg[lo];
+  const uint32_t lt = t - tt.tile_prefix[lo];
+  const uint32_t tps = tt.tiles_per_seg[lo];
   TileCoord c;
   c.item = lo;
-  if (launch.rank_major) {
+  if (tt.rank_major) {
     c.rank = lt / tps;
     c.chunk = lt - c.rank * tps;
   } else {
-    c.chunk = lt / launch.world;
-    c.rank = lt - c.chunk * launch.world;
+    c.chunk = lt / tt.world;
+    c.rank = lt - c.chunk * tt.world;
   }
-  c.rank += first_rank;
-  if (c.rank >= launch.world) c.rank -= launch.world;
+  c.rank += tt.first_rank;
+  if (c.rank >= tt.world) c.rank -= tt.world;
   return c;
 }
 
@@ -190,8 +204,8 @@ __device__ __forceinline__ void copy_any(uint8_t* d, const uint8_t* s, uint32_t 
 }
 
 __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
-  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch, t, launch.first_rank);
+  for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_bytes[c.item];
     const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
     const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride +
@@ -215,8 +229,8 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
 // ---- clear --------------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launch) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch, t, 0);
+  for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_bytes[c.item];
     const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
     uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.off[c.item] + in_seg;
@@ -367,8 +381,8 @@ template <class G, class A>
 __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launch) {
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
-  for (uint32_t t = blockIdx.x; t < launch.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch, t, 0);
+  for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_elems[c.item];
     const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
     const uint64_t g0 = (uint64_t)c.rank * seg + in_seg;  // element index in the full gradient
@@ -399,6 +413,97 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
       }
     } else {
       accum_any<G, A>(acc, grad, g0, grad_elems, left < kTileElems ? (uint32_t)left : kTileElems);
+    }
+  }
+}
+
+// ---- gather with cast ---------------------------------------------------------------------
+// dst[r*S + i] = narrow_D(widen_S(region_r[off + i])): the gather of shards kept in one dtype
+// (fp32 master copies) into a full parameter of another (bf16), in one pass.
+template <class S, class D>
+__device__ __forceinline__ void cast_one(uint8_t* d, const uint8_t* s, uint32_t i) {
+  typedef typename Codec<S>::raw_t sraw_t;
+  typedef typename Codec<D>::raw_t draw_t;
+  reinterpret_cast<draw_t*>(d)[i] = Codec<D>::narrow(Codec<S>::widen(reinterpret_cast<const sraw_t*>(s)[i]));
+}
+
+template <class S, class D>
+__device__ __forceinline__ void cast_any(uint8_t* d, const uint8_t* s, uint32_t n) {
+  typedef typename Quad<S>::vec_t svec_t;
+  typedef typename Quad<D>::vec_t dvec_t;
+  constexpr uint32_t kDstVecBytes = 4 * Codec<D>::kBytes;
+  const uint32_t tid = threadIdx.x;
+  uint32_t head = ((kDstVecBytes - (uint32_t)((uintptr_t)d & (kDstVecBytes - 1))) &
+                   (kDstVecBytes - 1)) / Codec<D>::kBytes;
+  if (head > n) head = n;
+  if (tid < head) cast_one<S, D>(d, s, tid);
+  const uint32_t nvec = (n - head) >> 2;
+  for (uint32_t v = tid; v < nvec; v += kThreads) {
+    const uint32_t i = head + 4 * v;
+    svec_t raw;
+    __builtin_memcpy(&raw, s + (size_t)i * Codec<S>::kBytes, sizeof(svec_t));
+    float f[4];
+    Quad<S>::widen(raw, f);
+    __builtin_nontemporal_store(Quad<D>::narrow(f),
+                                reinterpret_cast<dvec_t*>(d + (size_t)i * Codec<D>::kBytes));
+  }
+  const uint32_t done = head + 4 * nvec;
+  if (tid < n - done) cast_one<S, D>(d, s, done + tid);
+}
+
+template <class S, class D>
+__global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherLaunch launch) {
+  typedef typename Quad<S>::vec_t svec_t;
+  typedef typename Quad<D>::vec_t dvec_t;
+  for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch.tt, t);
+    const uint64_t seg = launch.seg_elems[c.item];
+    const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride +
+                       launch.src_off[c.item] + in_seg * Codec<S>::kBytes;
+    uint8_t* d = launch.dst[c.item] + ((uint64_t)c.rank * seg + in_seg) * Codec<D>::kBytes;
+    const uint64_t left = seg - in_seg;
+    if (left >= kTileElems && (((uintptr_t)s) & (sizeof(svec_t) - 1)) == 0 &&
+        (((uintptr_t)d) & (sizeof(dvec_t) - 1)) == 0) {
+      const svec_t* sp = reinterpret_cast<const svec_t*>(s) + threadIdx.x;
+      dvec_t* dp = reinterpret_cast<dvec_t*>(d) + threadIdx.x;
+      svec_t raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) raw[u] = __builtin_nontemporal_load(sp + u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        float f[4];
+        Quad<S>::widen(raw[u], f);
+        __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * kThreads);
+      }
+    } else {
+      cast_any<S, D>(d, s, left < kTileElems ? (uint32_t)left : kTileElems);
+    }
+  }
+}
+
+// ---- publish ------------------------------------------------------------------------------
+// One rank's accumulations at the end of a minibatch: acc[i] /= divisor in place (a correctly
+// rounded IEEE division, rounded to the accumulation dtype) and out[i] = narrow_O(acc[i]).
+template <class A, class O>
+__global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch launch) {
+  typedef typename Codec<A>::raw_t araw_t;
+  typedef typename Codec<O>::raw_t oraw_t;
+  for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
+    const TileCoord c = locate_tile(launch.tt, t);
+    const uint64_t seg = launch.seg_elems[c.item];
+    const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
+    araw_t* acc = reinterpret_cast<araw_t*>(launch.region + launch.acc_off[c.item]) + in_seg;
+    oraw_t* out = launch.out[c.item] ? reinterpret_cast<oraw_t*>(launch.out[c.item]) + in_seg : nullptr;
+    const uint64_t left = seg - in_seg;
+    const uint32_t n = left < kTileElems ? (uint32_t)left : kTileElems;
+    for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
+      araw_t raw = acc[i];
+      if (launch.divide) {
+        raw = Codec<A>::narrow(Codec<A>::widen(raw) / launch.divisor);
+        acc[i] = raw;
+      }
+      if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw));
     }
   }
 }
@@ -665,116 +770,6 @@ int odc_arena_locate(const odc_arena* a, const void* ptr, uint32_t* rank, uint64
 // ------------------------------------------------------------------------------------------------
 // launches
 // ------------------------------------------------------------------------------------------------
-int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uint32_t first_rank,
-               void* stream) {
-  DeviceGuard guard;
-  if (int rc = check_compute(a, guard)) return rc;
-  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
-  if (first_rank >= a->world)
-    return fail(ODC_ERR_INVALID, "first_rank %u >= world size %u", first_rank, a->world);
-  for (uint32_t i = 0; i < n_items; ++i) {
-    const odc_gather_item& it = items[i];
-    if (it.shard_bytes == 0) continue;
-    if (!it.dst) return fail(ODC_ERR_INVALID, "item %u: dst is NULL", i);
-    if (it.src_offset > a->bytes_per_rank || it.shard_bytes > a->bytes_per_rank - it.src_offset)
-      return fail(ODC_ERR_INVALID, "item %u: [%llu, +%llu) leaves the %llu byte rank region", i,
-                  (unsigned long long)it.src_offset, (unsigned long long)it.shard_bytes,
-                  (unsigned long long)a->bytes_per_rank);
-    const uint8_t* d0 = static_cast<const uint8_t*>(it.dst);
-    const uint8_t* d1 = d0 + it.shard_bytes * a->world;
-    const uint8_t* s0 = a->base + it.src_offset;
-    const uint8_t* s1 = a->base + (uint64_t)(a->world - 1) * a->rank_stride + it.src_offset + it.shard_bytes;
-    if (d0 < s1 && s0 < d1) {
-      // dst lies somewhere inside the arena span: refuse only a true overlap with a shard read
-      for (uint32_t r = 0; r < a->world; ++r) {
-        const uint8_t* rs0 = a->base + (uint64_t)r * a->rank_stride + it.src_offset;
-        if (d0 < rs0 + it.shard_bytes && rs0 < d1)
-          return fail(ODC_ERR_INVALID, "item %u: dst overlaps rank %u's shard", i, r);
-      }
-    }
-  }
-  const Options opt = options_snapshot();
-  uint32_t i = 0;
-  while (i < n_items) {
-    GatherLaunch L;
-    L.base = a->base;
-    L.rank_stride = a->rank_stride;
-    L.world = a->world;
-    L.first_rank = first_rank;
-    L.rank_major = opt.rank_major ? 1u : 0u;
-    uint32_t n = 0;
-    uint64_t tiles = 0;
-    for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
-      if (items[i].shard_bytes == 0) continue;
-      const uint64_t tps = (items[i].shard_bytes + kTileBytes - 1) / kTileBytes;
-      if (tps * a->world >= kMaxTilesPerLaunch)
-        return fail(ODC_ERR_INVALID, "item %u: shard of %llu bytes is too large for one launch", i,
-                    (unsigned long long)items[i].shard_bytes);
-      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
-      L.tile_prefix[n] = (uint32_t)tiles;
-      L.tiles_per_seg[n] = (uint32_t)tps;
-      L.dst[n] = static_cast<uint8_t*>(items[i].dst);
-      L.src_off[n] = items[i].src_offset;
-      L.seg_bytes[n] = items[i].shard_bytes;
-      tiles += tps * a->world;
-      ++n;
-    }
-    if (n == 0) continue;
-    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
-    L.n_items = n;
-    L.n_tiles = (uint32_t)tiles;
-    const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.n_tiles);
-    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
-  }
-  return ODC_OK;
-}
-
-int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* stream) {
-  DeviceGuard guard;
-  if (int rc = check_compute(a, guard)) return rc;
-  if (n_spans && !spans) return fail(ODC_ERR_INVALID, "spans is NULL");
-  for (uint32_t i = 0; i < n_spans; ++i) {
-    if (spans[i].offset > a->bytes_per_rank || spans[i].nbytes > a->bytes_per_rank - spans[i].offset)
-      return fail(ODC_ERR_INVALID, "span %u: [%llu, +%llu) leaves the %llu byte rank region", i,
-                  (unsigned long long)spans[i].offset, (unsigned long long)spans[i].nbytes,
-                  (unsigned long long)a->bytes_per_rank);
-  }
-  const Options opt = options_snapshot();
-  uint32_t i = 0;
-  while (i < n_spans) {
-    ClearLaunch L;
-    L.base = a->base;
-    L.rank_stride = a->rank_stride;
-    L.world = a->world;
-    L.rank_major = 0u;  // a write-only stream runs fastest with the ranks interleaved
-    uint32_t n = 0;
-    uint64_t tiles = 0;
-    for (; i < n_spans && n < (uint32_t)kMaxItems; ++i) {
-      if (spans[i].nbytes == 0) continue;
-      const uint64_t tps = (spans[i].nbytes + kTileBytes - 1) / kTileBytes;
-      if (tps * a->world >= kMaxTilesPerLaunch)
-        return fail(ODC_ERR_INVALID, "span %u: %llu bytes is too large for one launch", i,
-                    (unsigned long long)spans[i].nbytes);
-      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
-      L.tile_prefix[n] = (uint32_t)tiles;
-      L.tiles_per_seg[n] = (uint32_t)tps;
-      L.off[n] = spans[i].offset;
-      L.seg_bytes[n] = spans[i].nbytes;
-      tiles += tps * a->world;
-      ++n;
-    }
-    if (n == 0) continue;
-    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
-    L.n_items = n;
-    L.n_tiles = (uint32_t)tiles;
-    const uint32_t grid = grid_for(a, opt.clear_blocks_per_cu, L.n_tiles);
-    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
-  }
-  return ODC_OK;
-}
-
 }  // extern "C"
 
 namespace {
@@ -788,25 +783,217 @@ int dtype_bytes(int dt) {
   }
 }
 
-typedef void (*accum_fn)(const AccumLaunch);
+// Cuts items [*next, n_items) into one launch: at most kMaxItems non-empty items and fewer than
+// kMaxTilesPerLaunch tiles. units(i) is the item's per-rank size in tile units (0 = skip);
+// take(slot, i) copies item i's descriptor into slot `slot` of the launch. Returns the number of
+// items taken (0 when only empty items were left) or a negative status.
+template <class Units, class Take>
+int fill_tile_table(TileTable& tt, uint32_t world, uint32_t n_items, uint32_t* next,
+                    uint64_t tile_units, Units units, Take take) {
+  uint32_t n = 0;
+  uint64_t tiles = 0;
+  uint32_t i = *next;
+  for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
+    const uint64_t sz = units(i);
+    if (sz == 0) continue;
+    const uint64_t tps = (sz + tile_units - 1) / tile_units;
+    if (tps * world >= kMaxTilesPerLaunch)
+      return fail(ODC_ERR_INVALID, "item %u: %llu units per rank is too large for one launch", i,
+                  (unsigned long long)sz);
+    if (tiles + tps * world >= kMaxTilesPerLaunch) break;
+    tt.tile_prefix[n] = (uint32_t)tiles;
+    tt.tiles_per_seg[n] = (uint32_t)tps;
+    take(n, i);
+    tiles += tps * world;
+    ++n;
+  }
+  *next = i;
+  for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) tt.tile_prefix[k] = (uint32_t)tiles;
+  for (uint32_t k = n; k < (uint32_t)kMaxItems; ++k) tt.tiles_per_seg[k] = 1;
+  tt.world = world;
+  tt.n_items = n;
+  tt.n_tiles = (uint32_t)tiles;
+  return (int)n;
+}
 
-accum_fn pick_accum(int g, int a) {
-#define ODC_PAIR(GE, GT, AE, AT) if (g == GE && a == AE) return accum_kernel<GT, AT>;
-  ODC_PAIR(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_F32, f32_tag)
-  ODC_PAIR(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F32, f32_tag)
-  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F32, f32_tag)
-  ODC_PAIR(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_BF16, bf16_tag)
-  ODC_PAIR(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F16, f16_tag)
-  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_BF16, bf16_tag)
-  ODC_PAIR(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F16, f16_tag)
-#undef ODC_PAIR
+int check_rank_range(const odc_arena* a, const char* what, uint32_t i, uint64_t offset, uint64_t nbytes) {
+  if (offset > a->bytes_per_rank || nbytes > a->bytes_per_rank - offset)
+    return fail(ODC_ERR_INVALID, "%s %u: [%llu, +%llu) leaves the %llu byte rank region", what, i,
+                (unsigned long long)offset, (unsigned long long)nbytes,
+                (unsigned long long)a->bytes_per_rank);
+  return ODC_OK;
+}
+
+// dst [d0, d0 + world*seg_bytes) must not overlap any rank's source range at src_offset.
+int check_no_overlap(const odc_arena* a, uint32_t i, const void* dst, uint64_t dst_seg_bytes,
+                     uint64_t src_offset, uint64_t src_seg_bytes) {
+  const uint8_t* d0 = static_cast<const uint8_t*>(dst);
+  const uint8_t* d1 = d0 + dst_seg_bytes * a->world;
+  if (d1 <= a->base || d0 >= a->base + a->rank_stride * a->world) return ODC_OK;
+  for (uint32_t r = 0; r < a->world; ++r) {
+    const uint8_t* s0 = a->base + (uint64_t)r * a->rank_stride + src_offset;
+    if (d0 < s0 + src_seg_bytes && s0 < d1)
+      return fail(ODC_ERR_INVALID, "item %u: dst overlaps rank %u's shard", i, r);
+  }
+  return ODC_OK;
+}
+
+typedef void (*accum_fn)(const AccumLaunch);
+typedef void (*cast_gather_fn)(const CastGatherLaunch);
+typedef void (*publish_fn)(const PublishLaunch);
+
+#define ODC_FOR_EACH_DTYPE_PAIR(X)                    \
+  X(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_BF16, bf16_tag) \
+  X(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_F16, f16_tag)   \
+  X(ODC_DTYPE_BF16, bf16_tag, ODC_DTYPE_F32, f32_tag)   \
+  X(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_BF16, bf16_tag)   \
+  X(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F16, f16_tag)     \
+  X(ODC_DTYPE_F16, f16_tag, ODC_DTYPE_F32, f32_tag)     \
+  X(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_BF16, bf16_tag)   \
+  X(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F16, f16_tag)     \
+  X(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F32, f32_tag)
+
+accum_fn pick_accum(int g, int a) {  // (gradient dtype, accumulation dtype)
+#define X(E1, T1, E2, T2) if (g == E1 && a == E2) return accum_kernel<T1, T2>;
+  ODC_FOR_EACH_DTYPE_PAIR(X)
+#undef X
+  return nullptr;
+}
+
+cast_gather_fn pick_cast_gather(int s, int d) {  // (shard dtype, output dtype)
+#define X(E1, T1, E2, T2) if (s == E1 && d == E2) return cast_gather_kernel<T1, T2>;
+  ODC_FOR_EACH_DTYPE_PAIR(X)
+#undef X
+  return nullptr;
+}
+
+publish_fn pick_publish(int a, int o) {  // (accumulation dtype, output dtype)
+#define X(E1, T1, E2, T2) if (a == E1 && o == E2) return publish_kernel<T1, T2>;
+  ODC_FOR_EACH_DTYPE_PAIR(X)
+#undef X
   return nullptr;
 }
 
 }  // namespace
 
-extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
-                                      int grad_dtype, int acc_dtype, void* stream) {
+extern "C" {
+
+int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uint32_t first_rank,
+               void* stream) {
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
+  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
+  if (first_rank >= a->world)
+    return fail(ODC_ERR_INVALID, "first_rank %u >= world size %u", first_rank, a->world);
+  for (uint32_t i = 0; i < n_items; ++i) {
+    const odc_gather_item& it = items[i];
+    if (it.shard_bytes == 0) continue;
+    if (!it.dst) return fail(ODC_ERR_INVALID, "item %u: dst is NULL", i);
+    if (int rc = check_rank_range(a, "item", i, it.src_offset, it.shard_bytes)) return rc;
+    if (int rc = check_no_overlap(a, i, it.dst, it.shard_bytes, it.src_offset, it.shard_bytes)) return rc;
+  }
+  const Options opt = options_snapshot();
+  uint32_t next = 0;
+  while (next < n_items) {
+    GatherLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.first_rank = first_rank;
+    const int n = fill_tile_table(
+        L.tt, a->world, n_items, &next, kTileBytes, [&](uint32_t i) { return items[i].shard_bytes; },
+        [&](uint32_t slot, uint32_t i) {
+          L.dst[slot] = static_cast<uint8_t*>(items[i].dst);
+          L.src_off[slot] = items[i].src_offset;
+          L.seg_bytes[slot] = items[i].shard_bytes;
+        });
+    if (n < 0) return n;
+    if (n == 0) continue;
+    const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
+    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_items,
+                    int src_dtype, int dst_dtype, uint32_t first_rank, void* stream) {
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
+  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
+  if (first_rank >= a->world)
+    return fail(ODC_ERR_INVALID, "first_rank %u >= world size %u", first_rank, a->world);
+  const int sb = dtype_bytes(src_dtype), db = dtype_bytes(dst_dtype);
+  if (!sb || !db) return fail(ODC_ERR_INVALID, "unknown dtype code (src %d, dst %d)", src_dtype, dst_dtype);
+  const cast_gather_fn kernel = pick_cast_gather(src_dtype, dst_dtype);
+  if (!kernel) return fail(ODC_ERR_UNSUPPORTED, "gather from dtype %d into dtype %d is not implemented", src_dtype, dst_dtype);
+  for (uint32_t i = 0; i < n_items; ++i) {
+    const odc_gather_cast_item& it = items[i];
+    if (it.shard_elems == 0) continue;
+    if (!it.dst) return fail(ODC_ERR_INVALID, "item %u: dst is NULL", i);
+    if (it.shard_elems > a->bytes_per_rank / sb)
+      return fail(ODC_ERR_INVALID, "item %u: shard of %llu elements exceeds the rank region", i,
+                  (unsigned long long)it.shard_elems);
+    if (it.src_offset % sb || (uintptr_t)it.dst % db)
+      return fail(ODC_ERR_INVALID, "item %u: src_offset or dst is not aligned to its dtype", i);
+    if (int rc = check_rank_range(a, "item", i, it.src_offset, it.shard_elems * sb)) return rc;
+    if (int rc = check_no_overlap(a, i, it.dst, it.shard_elems * db, it.src_offset, it.shard_elems * sb)) return rc;
+  }
+  const Options opt = options_snapshot();
+  uint32_t next = 0;
+  while (next < n_items) {
+    CastGatherLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.first_rank = first_rank;
+    const int n = fill_tile_table(
+        L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
+        [&](uint32_t slot, uint32_t i) {
+          L.dst[slot] = static_cast<uint8_t*>(items[i].dst);
+          L.src_off[slot] = items[i].src_offset;
+          L.seg_elems[slot] = items[i].shard_elems;
+        });
+    if (n < 0) return n;
+    if (n == 0) continue;
+    const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* stream) {
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
+  if (n_spans && !spans) return fail(ODC_ERR_INVALID, "spans is NULL");
+  for (uint32_t i = 0; i < n_spans; ++i)
+    if (int rc = check_rank_range(a, "span", i, spans[i].offset, spans[i].nbytes)) return rc;
+  const Options opt = options_snapshot();
+  uint32_t next = 0;
+  while (next < n_spans) {
+    ClearLaunch L;
+    L.base = a->base;
+    L.rank_stride = a->rank_stride;
+    L.tt.rank_major = 0u;  // a write-only stream runs fastest with the ranks interleaved
+    L.tt.first_rank = 0;
+    const int n = fill_tile_table(
+        L.tt, a->world, n_spans, &next, kTileBytes, [&](uint32_t i) { return spans[i].nbytes; },
+        [&](uint32_t slot, uint32_t i) {
+          L.off[slot] = spans[i].offset;
+          L.seg_bytes[slot] = spans[i].nbytes;
+        });
+    if (n < 0) return n;
+    if (n == 0) continue;
+    const uint32_t grid = grid_for(a, opt.clear_blocks_per_cu, L.tt.n_tiles);
+    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
+                           int grad_dtype, int acc_dtype, void* stream) {
   DeviceGuard guard;
   if (int rc = check_compute(a, guard)) return rc;
   if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
@@ -828,10 +1015,7 @@ extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items,
     if (it.acc_offset % ab)
       return fail(ODC_ERR_INVALID, "item %u: acc_offset %llu is not aligned to the accumulation dtype", i,
                   (unsigned long long)it.acc_offset);
-    if (it.acc_offset > a->bytes_per_rank || it.shard_elems * ab > a->bytes_per_rank - it.acc_offset)
-      return fail(ODC_ERR_INVALID, "item %u: accumulation [%llu, +%llu) leaves the %llu byte rank region", i,
-                  (unsigned long long)it.acc_offset, (unsigned long long)(it.shard_elems * ab),
-                  (unsigned long long)a->bytes_per_rank);
+    if (int rc = check_rank_range(a, "item", i, it.acc_offset, it.shard_elems * ab)) return rc;
     if (it.grad_elems > it.shard_elems * a->world)
       return fail(ODC_ERR_INVALID, "item %u: grad_elems %llu > world_size * shard_elems = %llu", i,
                   (unsigned long long)it.grad_elems, (unsigned long long)(it.shard_elems * a->world));
@@ -840,38 +1024,80 @@ extern "C" int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items,
       return fail(ODC_ERR_INVALID, "item %u: grad pointer is not aligned to the gradient dtype", i);
   }
   const Options opt = options_snapshot();
-  uint32_t i = 0;
-  while (i < n_items) {
+  uint32_t next = 0;
+  while (next < n_items) {
     AccumLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.world = a->world;
-    L.rank_major = opt.rank_major ? 1u : 0u;
-    uint32_t n = 0;
-    uint64_t tiles = 0;
-    for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
-      if (items[i].shard_elems == 0) continue;
-      const uint64_t tps = (items[i].shard_elems + kTileElems - 1) / kTileElems;
-      if (tps * a->world >= kMaxTilesPerLaunch)
-        return fail(ODC_ERR_INVALID, "item %u: shard of %llu elements is too large for one launch", i,
-                    (unsigned long long)items[i].shard_elems);
-      if (tiles + tps * a->world >= kMaxTilesPerLaunch) break;
-      L.tile_prefix[n] = (uint32_t)tiles;
-      L.tiles_per_seg[n] = (uint32_t)tps;
-      L.grad[n] = static_cast<const uint8_t*>(items[i].grad);
-      L.grad_elems[n] = items[i].grad_elems;
-      L.acc_off[n] = items[i].acc_offset;
-      L.seg_elems[n] = items[i].shard_elems;
-      tiles += tps * a->world;
-      ++n;
-    }
+    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.first_rank = 0;
+    const int n = fill_tile_table(
+        L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
+        [&](uint32_t slot, uint32_t i) {
+          L.grad[slot] = static_cast<const uint8_t*>(items[i].grad);
+          L.grad_elems[slot] = items[i].grad_elems;
+          L.acc_off[slot] = items[i].acc_offset;
+          L.seg_elems[slot] = items[i].shard_elems;
+        });
+    if (n < 0) return n;
     if (n == 0) continue;
-    for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) L.tile_prefix[k] = (uint32_t)tiles;
-    L.n_items = n;
-    L.n_tiles = (uint32_t)tiles;
-    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.n_tiles);
+    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.tt.n_tiles);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;
 }
+
+int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint32_t n_items,
+                int acc_dtype, int out_dtype, float divisor, void* stream) {
+  DeviceGuard guard;
+  if (int rc = check_compute(a, guard)) return rc;
+  if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
+  if (rank >= a->world) return fail(ODC_ERR_INVALID, "rank %u >= world size %u", rank, a->world);
+  const int ab = dtype_bytes(acc_dtype), ob = dtype_bytes(out_dtype);
+  if (!ab || !ob) return fail(ODC_ERR_INVALID, "unknown dtype code (acc %d, out %d)", acc_dtype, out_dtype);
+  if (!(divisor == divisor) || divisor == 0.0f) return fail(ODC_ERR_INVALID, "divisor must be a non-zero number");
+  const publish_fn kernel = pick_publish(acc_dtype, out_dtype);
+  if (!kernel) return fail(ODC_ERR_UNSUPPORTED, "publish from dtype %d into dtype %d is not implemented", acc_dtype, out_dtype);
+  uint8_t* region = a->base + (uint64_t)rank * a->rank_stride;
+  for (uint32_t i = 0; i < n_items; ++i) {
+    const odc_publish_item& it = items[i];
+    if (it.elems == 0) continue;
+    if (it.elems > a->bytes_per_rank / ab)
+      return fail(ODC_ERR_INVALID, "item %u: %llu elements exceed the rank region", i, (unsigned long long)it.elems);
+    if (it.acc_offset % ab || (uintptr_t)it.out % ob)
+      return fail(ODC_ERR_INVALID, "item %u: acc_offset or out is not aligned to its dtype", i);
+    if (int rc = check_rank_range(a, "item", i, it.acc_offset, it.elems * ab)) return rc;
+    if (it.out) {
+      const uint8_t* o0 = static_cast<const uint8_t*>(it.out);
+      const uint8_t* s0 = region + it.acc_offset;
+      if (o0 < s0 + it.elems * ab && s0 < o0 + it.elems * ob)
+        return fail(ODC_ERR_INVALID, "item %u: out overlaps the accumulation it is published from", i);
+    }
+  }
+  const Options opt = options_snapshot();
+  uint32_t next = 0;
+  while (next < n_items) {
+    PublishLaunch L;
+    L.region = region;
+    L.divisor = divisor;
+    L.divide = divisor != 1.0f;
+    L.tt.rank_major = 1u;
+    L.tt.first_rank = 0;
+    const int n = fill_tile_table(
+        L.tt, 1u, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].elems; },
+        [&](uint32_t slot, uint32_t i) {
+          L.out[slot] = static_cast<uint8_t*>(items[i].out);
+          L.acc_off[slot] = items[i].acc_offset;
+          L.seg_elems[slot] = items[i].elems;
+        });
+    if (n < 0) return n;
+    if (n == 0) continue;
+    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.tt.n_tiles);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    ODC_HIP_TRY(hipGetLastError());
+  }
+  return ODC_OK;
+}
+
+}  // extern "C"

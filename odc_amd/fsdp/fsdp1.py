@@ -22,7 +22,7 @@ import torch
 import torch.nn.functional as F
 
 import odc_amd
-from odc_amd.primitives.utils import comm_stream_section, group_size
+from odc_amd.primitives.utils import group_size
 
 logger = logging.getLogger(__name__)
 
@@ -60,20 +60,17 @@ def get_shard(tensor: torch.Tensor, rank: int, world_size: int):
 
 
 def all_gather_flat_param(padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=None):
-    """Gather the padded flat parameter. When ``param_dtype`` differs from the shard dtype the
-    gather runs in the shard dtype into a temporary and is then cast, as the reference must
-    because a peer may not have produced its low-precision shard yet (fsdp1.py:199-223)."""
+    """Gather the padded flat parameter. The shards stay in their own dtype (a peer may not have
+    produced a low-precision copy yet: that is why the reference gathers in the shard dtype into
+    a temporary and casts afterwards, fsdp1.py:199-223); when the output dtype differs, the
+    conversion happens inside the gather kernel."""
     expected = sharded_flat_param.numel() * group_size(pg)
     assert (
         padded_unsharded_flat_param.numel() == expected
     ), f"Expects {expected} numel but got {padded_unsharded_flat_param.numel()}"
     if padded_unsharded_flat_param.dtype != sharded_flat_param.dtype:
         assert param_dtype in (None, padded_unsharded_flat_param.dtype)
-        tmp = torch.empty_like(padded_unsharded_flat_param, dtype=sharded_flat_param.dtype)
-        gather_service.gather_into_tensor(tmp, sharded_flat_param, pg)
-        padded_unsharded_flat_param.copy_(tmp)
-    else:
-        gather_service.gather_into_tensor(padded_unsharded_flat_param, sharded_flat_param, pg)
+    gather_service.gather_into_tensor(padded_unsharded_flat_param, sharded_flat_param, pg)
     return padded_unsharded_flat_param
 
 
@@ -122,13 +119,20 @@ def pre_optimizer_step(fsdp_module):
         raise NotImplementedError("hybrid sharding needs a second node; not part of this build")
     service = get_reduction_service()
     factor = getattr(fsdp_module, "_gradient_postdivide_factor", 1.0)
-    with comm_stream_section():
-        for key in service.accumulations:
-            _div_if_needed(service.get_accumulation(key), factor)
-    for handle in fsdp_module._all_handles:
-        handle.flat_param.grad = service.get_accumulation(id(handle.flat_param)).to(
-            handle.flat_param.dtype
-        )
+    divisor = factor if factor is not None and factor > 1 else 1.0  # `_div_if_needed`
+    handles = list(fsdp_module._all_handles)
+    by_dtype = {}
+    for handle in handles:
+        by_dtype.setdefault(handle.flat_param.dtype, []).append(handle)
+    published = set()
+    for dtype, group in by_dtype.items():
+        keys = [id(h.flat_param) for h in group]
+        for handle, grad in zip(group, service.publish(keys, out_dtype=dtype, divisor=divisor)):
+            handle.flat_param.grad = grad
+        published.update(keys)
+    rest = [k for k in service.accumulations if k not in published]
+    if rest and divisor != 1.0:  # the reference divides every accumulation, handle or not
+        service.publish(rest, divisor=divisor)
 
 
 def pre_minibatch_start(_fsdp_module):

@@ -34,7 +34,6 @@ from odc_amd.primitives.gather import GatherService
 from odc_amd.primitives.scatter_accumulate import ReductionService
 from odc_amd.primitives.utils import (
     SymmBufferRegistry,
-    comm_stream_section,
     finalize_distributed,
     get_rank,
     group_size,
@@ -121,18 +120,21 @@ class ParamGroup:
     def unshard(self, fused: bool = True) -> List[torch.Tensor]:
         W = self.world_size
         device = self.symm_buffer.device
-        padded = [torch.empty(W * n, dtype=self.dtype, device=device) for n in self.shard_numels]
+        out_dtype = self.param_dtype or self.dtype
         gather = get_gather_service()
         if fused:
+            # straight into per-parameter buffers, converted to the compute dtype on the way
+            padded = [torch.empty(W * n, dtype=out_dtype, device=device) for n in self.shard_numels]
             gather.gather_slices(padded, self.symm_buffer, self.offsets, self.shard_numels, self.pg)
         else:
+            padded = [torch.empty(W * n, dtype=self.dtype, device=device) for n in self.shard_numels]
             ag = torch.empty(W * self.total_shard_numel, dtype=self.dtype, device=device)
             gather.gather_into_tensor(ag, self.symm_buffer, self.pg)
             torch.split_with_sizes_copy(
                 ag.view(W, -1), self.shard_numels, dim=1, out=[t.view(W, -1) for t in padded]
             )
-        if self.param_dtype is not None and self.param_dtype != self.dtype:
-            padded = [t.to(self.param_dtype) for t in padded]  # fsdp2.py:341-343
+            if out_dtype != self.dtype:
+                padded = [t.to(out_dtype) for t in padded]  # fsdp2.py:341-343
         self._unsharded = [
             t.view(-1, *shape[1:])[: shape[0]] for t, shape in zip(padded, self.shapes)
         ]
@@ -176,12 +178,10 @@ class ParamGroup:
         if not self._reduced:
             return None  # no microbatch touched this group in this minibatch (fsdp2.py:797-801)
         self._reduced = False
-        reduce_output = get_reduction_service().get_accumulation(id(self))
-        with comm_stream_section():
-            if self.reduce_op == "avg":
-                reduce_output /= self.world_size
-            if reduce_output.dtype != self.dtype:
-                reduce_output = reduce_output.to(self.dtype)
+        divisor = float(self.world_size) if self.reduce_op == "avg" else 1.0
+        (reduce_output,) = get_reduction_service().publish(
+            [id(self)], out_dtype=self.dtype, divisor=divisor
+        )
         rank = get_rank()
         grads = []
         for p, shape in enumerate(self.shapes):

@@ -22,6 +22,7 @@ from odc_amd.primitives.utils import (
     get_rank,
     get_world,
     group_size,
+    native_dtype,
 )
 
 logger = logging.getLogger(__name__)
@@ -43,32 +44,47 @@ class GatherService:
         self, output_tensors: Sequence[Tensor], input_tensors: Sequence[Tensor], pg
     ) -> None:
         """Multi-tensor form: every (output, input) pair of the lists in ONE launch (per 32
-        pairs). Equivalent to calling ``gather_into_tensor`` pair by pair."""
+        pairs). Equivalent to calling ``gather_into_tensor`` pair by pair. When the outputs'
+        dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)
         world = get_world()
         W = group_size(pg)
         assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
         registry = SymmBufferRegistry.get_instance()
         pairs = [(o, i) for o, i in zip(output_tensors, input_tensors) if i.numel() or o.numel()]
-        items = (_native.GatherItem * max(len(pairs), 1))()
+        if not pairs:
+            return
+        src_dtype, dst_dtype = pairs[0][1].dtype, pairs[0][0].dtype
+        cast = src_dtype != dst_dtype
+        items = ((_native.GatherCastItem if cast else _native.GatherItem) * len(pairs))()
         for i, (out, inp) in enumerate(pairs):
             assert out.is_cuda and inp.is_cuda, "gather runs on the GPU only"
-            assert out.dtype == inp.dtype, f"{out.dtype=} != {inp.dtype=}"
+            assert (inp.dtype, out.dtype) == (src_dtype, dst_dtype), "one launch takes one dtype pair"
             assert out.is_contiguous() and inp.is_contiguous()
             assert (
                 out.numel() == W * inp.numel()
             ), f"output numel {out.numel()} != {W} * shard numel {inp.numel()}"
             items[i].dst = out.data_ptr()
             items[i].src_offset = registry.symmetric_offset_of(inp)
-            items[i].shard_bytes = inp.numel() * inp.element_size()
+            if cast:
+                items[i].shard_elems = inp.numel()
+            else:
+                items[i].shard_bytes = inp.numel() * inp.element_size()
 
+        lib = _native.load()
         with comm_stream_section() as comm:
-            _native.check(
-                _native.load().odc_gather(
-                    world.arena.handle, items, len(pairs), get_rank(),
-                    ctypes.c_void_p(comm.cuda_stream),
+            stream = ctypes.c_void_p(comm.cuda_stream)
+            if cast:
+                # shards kept in one dtype (fp32 master copies), full parameter wanted in another
+                # (bf16): converted on the way instead of gathered and then cast
+                # (odc/fsdp/fsdp1.py:199-223, odc/fsdp/fsdp2.py:341-343)
+                status = lib.odc_gather_cast(
+                    world.arena.handle, items, len(pairs), native_dtype(src_dtype),
+                    native_dtype(dst_dtype), get_rank(), stream,
                 )
-            )
+            else:
+                status = lib.odc_gather(world.arena.handle, items, len(pairs), get_rank(), stream)
+            _native.check(status)
 
     def gather_slices(
         self,

@@ -214,6 +214,47 @@ class ReductionService:
             raise KeyError(key)
         return SymmBufferRegistry.get_instance().get_symm_buffer(self._acc_key(key))
 
+    def publish(self, keys: Sequence, out_dtype=None, divisor: float = 1.0):
+        """End-of-minibatch pass over the calling rank's accumulations ``keys``, in one launch:
+        ``acc /= divisor`` in place (skipped for 1) and, when ``out_dtype`` differs from the
+        accumulation dtype, a cast copy. Returns one tensor per key: the cast copy, or the live
+        accumulation itself when no cast is needed (as ``acc.to(dtype)`` does).
+        ``odc/fsdp/fsdp1.py:324-335``; ``odc/fsdp/fsdp2.py:846-847,897-899``."""
+        if not keys:
+            return []
+        registry = SymmBufferRegistry.get_instance()
+        items = (_native.PublishItem * len(keys))()
+        results, acc_dtype = [], None
+        for i, key in enumerate(keys):
+            offset, shape, dtype = registry.offsets[self._acc_key(key)]
+            assert acc_dtype in (None, dtype), "one launch takes one accumulation dtype"
+            acc_dtype = dtype
+            acc = self.get_accumulation(key)
+            items[i].acc_offset = offset
+            items[i].elems = shape[0]
+            if out_dtype is None or out_dtype == dtype:
+                items[i].out = None
+                results.append(acc)
+            else:
+                out = torch.empty(shape, dtype=out_dtype, device=acc.device)
+                items[i].out = out.data_ptr()
+                results.append(out)
+        target = acc_dtype if out_dtype is None else out_dtype
+        with comm_stream_section() as comm:
+            _native.check(
+                _native.load().odc_publish(
+                    get_world().arena.handle,
+                    get_rank(),
+                    items,
+                    len(items),
+                    native_dtype(acc_dtype),
+                    native_dtype(target),
+                    float(divisor),
+                    ctypes.c_void_p(comm.cuda_stream),
+                )
+            )
+        return results
+
     def get_peer_accumulations(self, key):
         """All W ranks' accumulation buffers for ``key`` (virtual-world convenience)."""
         return SymmBufferRegistry.get_instance().peer_tensors[self._acc_key(key)]

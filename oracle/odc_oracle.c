@@ -99,3 +99,7 @@ void oracle_widen_bf16(float* out, const uint16_t* in, uint64_t n) {
 void oracle_widen_f16(float* out, const uint16_t* in, uint64_t n) {
   for (uint64_t i = 0; i < n; ++i) out[i] = widen_f16(in[i]);
 }
+
+void oracle_narrow_bf16(uint16_t* out, const float* in, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) out[i] = narrow_bf16(in[i]);
+}

@@ -9,6 +9,9 @@ Every function restates, with stock torch CPU ops, what the reference computes f
 repository (sail-sg/odc) or, where marked ``torch/``, in the PyTorch the reference patches.
 
 How each function is pinned (tests/test_oracle.py):
+  gather_cast               fp32->bf16 against the C restatement's integer round-to-nearest-even
+                            on random values, ties and every exponent; widening casts are exact.
+  fsdp1_publish / fsdp2_average   torch CPU div_ against numpy float32 division.
   gather_into_tensor        closed-form ``i + 2r`` pattern of examples/all_gather.py:80-84,121-125;
                             brute-force Python loops on tiny inputs; sentinel bytes around dst.
   scatter_accumulate        closed forms (ones x M == M, powers of two, +0 + -0 == +0, Inf/NaN);
@@ -52,6 +55,14 @@ def gather_into_tensor(
 def gather(shards: Sequence[torch.Tensor]) -> torch.Tensor:
     """The same result as a fresh tensor: ``torch.cat`` of the W shards."""
     return torch.cat([s.reshape(-1) for s in shards])
+
+
+def gather_cast(shards: Sequence[torch.Tensor], dtype: torch.dtype) -> torch.Tensor:
+    """Gather in the shards' dtype, then convert the full parameter: odc/fsdp/fsdp1.py:199-223
+    (``padded_unsharded_flat_param.copy_(…orig_dtype)``) and odc/fsdp/fsdp2.py:341-343
+    (``_to_dtype_if_needed(all_gather_output, param_dtype)``). torch's conversion rounds to
+    nearest even."""
+    return gather(shards).to(dtype)
 
 
 # --------------------------------------------------------------------------------------------

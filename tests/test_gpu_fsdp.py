@@ -111,10 +111,5 @@ def test_fsdp2_group_layout(make_world, W, fused, dtype):
             wantv = oracle.fsdp2_grad_views(oracle.fsdp2_average(accs[r].clone(), W).to(dtype), shapes, W, r)
             for p, (a, b) in enumerate(zip(got, wantv)):
                 assert tuple(a.shape) == tuple(b.shape), f"rank {r} param {p}"
-                if W & (W - 1) == 0:
-                    assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
-                else:
-                    # the averaging is torch's own `/=` on the device, which multiplies by the
-                    # rounded reciprocal of a scalar divisor: exact only for powers of two
-                    torch.testing.assert_close(a.cpu(), b, rtol=1e-6, atol=0)
+                assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
     assert set(fsdp2.get_symm_buffer_memory_breakdown()) >= {"fsdp_params", "accumulation"}

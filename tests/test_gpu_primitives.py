@@ -199,3 +199,71 @@ def test_hip_graph_capture_and_replay(make_world):
         assert_bit_equal(out, oracle.gather(shards), f"replay {replay}: gather")
         for r, acc in enumerate(reduction.get_peer_accumulations("p")):
             assert_bit_equal(acc, want_acc[r], f"replay {replay}: accumulation of rank {r}")
+
+
+@pytest.mark.parametrize("src_dtype,dst_dtype", [
+    (torch.float32, torch.bfloat16), (torch.float32, torch.float16), (torch.bfloat16, torch.float32),
+    (torch.float16, torch.float32), (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16),
+])
+@pytest.mark.parametrize("W,S", [(1, 3), (8, 4096), (8, 4099), (12, 33_337), (3, 70_001), (64, 64)])
+def test_gather_with_cast(make_world, src_dtype, dst_dtype, W, S):
+    """Shards in one dtype gathered into a full parameter of another in one pass equal the
+    reference's gather-then-cast."""
+    group = make_world(W, 4 << 20)
+    gather, _, registry = services()
+    g = torch.Generator().manual_seed(S + W)
+    shards = [(torch.randn(S, generator=g) * 10.0 ** (r % 5 - 2)).to(src_dtype) for r in range(W)]
+    src = put_shards(registry, "p", shards, group)
+    buf = torch.full((W * S + 16,), 7.0, dtype=dst_dtype, device="cuda")
+    dst = buf[5 : 5 + W * S]  # odd element offset: unaligned destination
+    gather.gather_into_tensor(dst, src, group)
+    assert_bit_equal(dst, oracle.gather_cast(shards, dst_dtype), f"{src_dtype}->{dst_dtype} W={W} S={S}")
+    assert (buf[:5] == 7).all() and (buf[5 + W * S :] == 7).all()
+
+
+def test_gather_with_cast_special_values(make_world):
+    W = 4
+    group = make_world(W, 4 << 20)
+    gather, _, registry = services()
+    ties = (2.0 ** torch.arange(-149, 127, dtype=torch.float64)).float() * 1.00390625
+    vals = torch.cat([ties, -ties, torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 3.4e38, -3.4e38, 1e-45, float("nan")])])
+    vals = torch.cat([vals, torch.zeros((-vals.numel()) % W)])
+    shards = list(vals.view(W, -1))
+    src = put_shards(registry, "v", shards, group)
+    out = torch.empty(vals.numel(), dtype=torch.bfloat16, device="cuda")
+    gather.gather_into_tensor(out, src, group)
+    want = oracle.gather_cast(shards, torch.bfloat16)
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out.cpu()), nan)
+    assert_bit_equal(out.cpu()[~nan], want[~nan], "ties, overflow to inf, denormals, signed zero")
+
+
+@pytest.mark.parametrize("divisor", [1.0, 8.0, 12.0, 3.0])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_publish_divides_in_place_and_casts(make_world, divisor, out_dtype):
+    """acc /= divisor with a correctly rounded division (bit-equal to torch CPU div_) and the cast
+    copy, for two keys in one launch, on a rank other than 0."""
+    from odc_amd import ReductionService, virtual_rank
+
+    W = 4
+    group = make_world(W, 4 << 20)
+    reduction = ReductionService(accumulation_dtype=torch.float32)
+    g = torch.Generator().manual_seed(int(divisor))
+    sizes = {"a": 10_007, "b": 4096}
+    want = {k: [torch.zeros(n) for _ in range(W)] for k, n in sizes.items()}
+    for k, n in sizes.items():
+        grad = torch.randn(W * n, generator=g).bfloat16()
+        reduction.scatter_accumulate(k, grad.cuda(), group)
+        oracle.scatter_accumulate(want[k], grad)
+    with virtual_rank(2):
+        outs = reduction.publish(["a", "b"], out_dtype=out_dtype, divisor=divisor)
+        reduction.sync(group)
+        for k, out in zip(sizes, outs):
+            acc = want[k][2].clone()
+            expect = oracle.fsdp1_publish(acc, divisor, out_dtype)
+            assert_bit_equal(out, expect, f"published {k}")
+            assert_bit_equal(reduction.get_accumulation(k), acc, f"accumulation {k} divided in place")
+            if out_dtype == torch.float32:
+                assert out.data_ptr() == reduction.get_accumulation(k).data_ptr()  # no copy, like .to()
+    for r in (0, 1, 3):  # other ranks untouched
+        assert_bit_equal(reduction.get_peer_accumulations("a")[r], want["a"][r], f"rank {r}")

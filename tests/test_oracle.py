@@ -20,8 +20,7 @@ ORACLE_DIR = Path(oracle.__file__).resolve().parent
 @pytest.fixture(scope="module")
 def c_oracle():
     lib_path = ORACLE_DIR / "libodc_oracle.so"
-    if not lib_path.exists():
-        subprocess.run(["make", "-C", str(ORACLE_DIR)], check=True)
+    subprocess.run(["make", "-C", str(ORACLE_DIR)], check=True, capture_output=True)
     lib = ctypes.CDLL(str(lib_path))
     lib.oracle_gather.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint32, ctypes.c_uint64]
     lib.oracle_scatter_accumulate_f32.argtypes = [
@@ -30,6 +29,7 @@ def c_oracle():
         ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint64]
     lib.oracle_widen_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
     lib.oracle_widen_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
+    lib.oracle_narrow_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
     return lib
 
 
@@ -83,6 +83,39 @@ def test_gather_is_a_byte_copy_for_every_bf16_pattern():
     allbits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
     shards = list(allbits.view(4, -1))
     assert torch.equal(_bits(oracle.gather(shards)), _bits(allbits))
+
+
+def test_gather_cast_rounds_to_nearest_even(c_oracle):
+    g = torch.Generator().manual_seed(17)
+    vals = torch.cat([
+        torch.randn(100_000, generator=g),
+        torch.randn(10_000, generator=g) * 1e-30, torch.randn(10_000, generator=g) * 1e30,
+        torch.tensor([1.0 + 2.0**-8, 1.0078125 + 2.0**-8, -(1.0 + 2.0**-8), 3.3895e38, 3.4e38, 1e-45, -0.0, 0.0,
+                      float("inf"), -float("inf")]),
+        (2.0 ** torch.arange(-149, 128, dtype=torch.float64)).float() * 1.00390625,  # ties at every exponent
+    ])
+    vals = torch.cat([vals, torch.zeros((-vals.numel()) % 4)])
+    shards = list(vals.view(4, -1))
+    got = oracle.gather_cast(shards, torch.bfloat16)
+    want = torch.empty(vals.numel(), dtype=torch.int16)
+    c_oracle.oracle_narrow_bf16(want.data_ptr(), vals.data_ptr(), vals.numel())
+    assert torch.equal(_bits(got), want)
+    assert got[100_000 + 20_000].item() == 1.0 and got[100_000 + 20_001].item() == 1.015625  # ties to even
+    # widening is exact
+    b = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    wide = oracle.gather_cast(list(b.view(8, -1)), torch.float32)
+    ok = ~torch.isnan(wide)
+    assert torch.equal(_bits(wide[ok]), (b.view(torch.int16).to(torch.int32) << 16)[ok])
+
+
+def test_division_matches_numpy_float32():
+    g = torch.Generator().manual_seed(19)
+    acc = torch.randn(50_000, generator=g) * 1e-2
+    for W in (1, 2, 3, 7, 8, 12, 64):
+        want = torch.from_numpy(acc.numpy() / np.float32(W))
+        assert torch.equal(_bits(oracle.fsdp2_average(acc.clone(), W)), _bits(want))
+        got = oracle.fsdp1_publish(acc.clone(), float(W), torch.bfloat16)
+        assert torch.equal(_bits(got), _bits(want.bfloat16() if W > 1 else acc.bfloat16()))
 
 
 # ---- scatter-accumulate ------------------------------------------------------------------------
