@@ -15,6 +15,7 @@ launch stream, the CPU oracle timed on the host cores, and the parity verdict.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import statistics
@@ -192,15 +193,26 @@ def main():
     # The services launch on the comm stream (as the reference does). Making it the current
     # stream here removes the stream joins from between the event pairs, so that each pair
     # brackets exactly one kernel.
+    # A full Python garbage collection (tens of ms with torch imported) landing inside the timed
+    # loop would stall the launches while an event pair is open: collect now, then keep the
+    # collector off until the loop is done.
+    gc.collect()
+    gc.disable()
     with torch.cuda.stream(comm):
         for i in range(args.warmup):
             step(i, record=False)
         torch.cuda.synchronize()
+        host_step = []
         t0 = time.perf_counter()
         for i in range(args.steps):
+            ts = time.perf_counter()
             step(i, record=True)
+            host_step.append(time.perf_counter() - ts)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
+        if os.environ.get("ODC_BENCH_DEBUG"):
+            print("host ms per step:", [round(x * 1e3, 3) for x in host_step], file=sys.stderr)
+    gc.enable()
 
     if args.calibrate:
         a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
@@ -208,10 +220,16 @@ def main():
         b.copy_(a)
         torch.cuda.synchronize()
 
+    def launch_ms(pairs):
+        return [a.elapsed_time(b) for a, b in pairs]
+
     def mean_ms(pairs):
-        return statistics.fmean(a.elapsed_time(b) for a, b in pairs) if pairs else None
+        return statistics.fmean(launch_ms(pairs)) if pairs else None
 
     g_ms, a_ms, c_ms = mean_ms(gather_events), mean_ms(accum_events), mean_ms(clear_events)
+    if os.environ.get("ODC_BENCH_DEBUG"):
+        print("gather ms per launch:", [round(x, 3) for x in launch_ms(gather_events)], file=sys.stderr)
+        print("accum ms per launch:", [round(x, 3) for x in launch_ms(accum_events)], file=sys.stderr)
     accum_gbps = 10 * N / (a_ms * 1e-3) / 1e9
     gather_gbps = 4 * N / (g_ms * 1e-3) / 1e9
     value = args.steps * 14 * N / elapsed / 1e9
@@ -243,6 +261,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(("accum", args.layout, W)),
             "algorithmic_bytes": 10 * N,
             "avg_launch_ms": round(a_ms, 5),
+            "min_launch_ms": round(min(launch_ms(accum_events)), 5),
+            "max_launch_ms": round(max(launch_ms(accum_events)), 5),
         },
         "roofline_gather": {
             "kernel": "gather_kernel",
@@ -254,6 +274,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(("gather", args.layout, W)),
             "algorithmic_bytes": 4 * N,
             "avg_launch_ms": round(g_ms, 5),
+            "min_launch_ms": round(min(launch_ms(gather_events)), 5),
+            "max_launch_ms": round(max(launch_ms(gather_events)), 5),
         },
         "clear": {"avg_launch_ms": round(c_ms, 5) if c_ms else None,
                   "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},

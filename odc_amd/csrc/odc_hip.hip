@@ -227,6 +227,7 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
 }
 
 // ---- clear --------------------------------------------------------------------------------
+// Plain (not nontemporal) stores: for a write-only stream they measure ~3 % faster here.
 __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launch) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launc
     if (left >= kTileBytes && (((uintptr_t)d) & 15u) == 0) {
       u32x4* dv = reinterpret_cast<u32x4*>(d) + threadIdx.x;
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(zero, dv + u * kThreads);
+      for (int u = 0; u < kUnroll; ++u) dv[u * kThreads] = zero;
     } else {
       uint32_t n = left < kTileBytes ? (uint32_t)left : kTileBytes;
       const uint32_t tid = threadIdx.x;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launc
       n -= head;
       const uint32_t nvec = n >> 4;
       for (uint32_t v = tid; v < nvec; v += kThreads)
-        __builtin_nontemporal_store(zero, reinterpret_cast<u32x4*>(d) + v);
+        reinterpret_cast<u32x4*>(d)[v] = zero;
       const uint32_t tail = n & 15u;
       if (tid < tail) d[(size_t)nvec * 16 + tid] = 0;
     }
