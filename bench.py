@@ -108,31 +108,27 @@ def main():
     torch.cuda.synchronize()
 
     comm = get_comm_stream()
-    gather_events, accum_events, clear_events = [], [], []
+    # One event after every launch of the timed region (plus one at its start): launch k's
+    # duration is the time between marks k and k+1, all recorded on the launch stream.
+    marks = []
+
+    def mark(label):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(comm)
+        marks.append((label, ev))
 
     def step(i, record):
         m = i % MICROBATCHES
         if m == 0:
-            if record:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(comm)
             reduction.clear_accumulations()
             if record:
-                e1.record(comm)
-                clear_events.append((e0, e1))
-        if record:
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(comm)
+                mark("clear")
         gather.gather_into_tensors(outs, shard_locals, group)
         if record:
-            e1.record(comm)
-            gather_events.append((e0, e1))
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(comm)
+            mark("gather")
         reduction.scatter_accumulate_multi(keys, grads[m], group)
         if record:
-            e1.record(comm)
-            accum_events.append((e0, e1))
+            mark("accum")
 
     # ---- parity + CPU baseline: one full minibatch against the oracle -------------------------
     cpu_baseline = None
@@ -203,6 +199,7 @@ def main():
             step(i, record=False)
         torch.cuda.synchronize()
         host_step = []
+        mark("start")
         t0 = time.perf_counter()
         for i in range(args.steps):
             ts = time.perf_counter()
@@ -220,16 +217,17 @@ def main():
         b.copy_(a)
         torch.cuda.synchronize()
 
-    def launch_ms(pairs):
-        return [a.elapsed_time(b) for a, b in pairs]
+    durations = {"clear": [], "gather": [], "accum": []}
+    for (_, before), (label, after) in zip(marks, marks[1:]):
+        durations[label].append(before.elapsed_time(after))
 
-    def mean_ms(pairs):
-        return statistics.fmean(launch_ms(pairs)) if pairs else None
+    def mean_ms(label):
+        return statistics.fmean(durations[label]) if durations[label] else None
 
-    g_ms, a_ms, c_ms = mean_ms(gather_events), mean_ms(accum_events), mean_ms(clear_events)
+    g_ms, a_ms, c_ms = mean_ms("gather"), mean_ms("accum"), mean_ms("clear")
     if os.environ.get("ODC_BENCH_DEBUG"):
-        print("gather ms per launch:", [round(x, 3) for x in launch_ms(gather_events)], file=sys.stderr)
-        print("accum ms per launch:", [round(x, 3) for x in launch_ms(accum_events)], file=sys.stderr)
+        print("gather ms per launch:", [round(x, 3) for x in durations["gather"]], file=sys.stderr)
+        print("accum ms per launch:", [round(x, 3) for x in durations["accum"]], file=sys.stderr)
     accum_gbps = 10 * N / (a_ms * 1e-3) / 1e9
     gather_gbps = 4 * N / (g_ms * 1e-3) / 1e9
     value = args.steps * 14 * N / elapsed / 1e9
@@ -261,8 +259,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(("accum", args.layout, W)),
             "algorithmic_bytes": 10 * N,
             "avg_launch_ms": round(a_ms, 5),
-            "min_launch_ms": round(min(launch_ms(accum_events)), 5),
-            "max_launch_ms": round(max(launch_ms(accum_events)), 5),
+            "min_launch_ms": round(min(durations["accum"]), 5),
+            "max_launch_ms": round(max(durations["accum"]), 5),
         },
         "roofline_gather": {
             "kernel": "gather_kernel",
@@ -274,8 +272,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(("gather", args.layout, W)),
             "algorithmic_bytes": 4 * N,
             "avg_launch_ms": round(g_ms, 5),
-            "min_launch_ms": round(min(launch_ms(gather_events)), 5),
-            "max_launch_ms": round(max(launch_ms(gather_events)), 5),
+            "min_launch_ms": round(min(durations["gather"]), 5),
+            "max_launch_ms": round(max(durations["gather"]), 5),
         },
         "clear": {"avg_launch_ms": round(c_ms, 5) if c_ms else None,
                   "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},
