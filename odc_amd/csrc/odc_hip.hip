@@ -177,83 +177,135 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable& tt, uint32_t t
   return c;
 }
 
-__device__ __forceinline__ u32x4 load16_unaligned(const uint8_t* p) {
-  u32x4 v;
-  __builtin_memcpy(&v, p, 16);
-  return v;
+// Tile geometry shared by all streaming kernels. A rank segment of `n` units (bytes, or
+// elements) whose written side starts at address D is cut as
+//     head  : the units before the first 16-byte (vector) boundary of D,
+//     body  : nvec whole vectors, written with aligned 128-bit (64-bit for 16-bit outputs) stores,
+//     tail  : what is left after the last whole vector.
+// Tile c owns body vectors [c*kTileVecs, (c+1)*kTileVecs); tile 0 also does the head, and the
+// tile holding the last body vector (tile 0 when there is none) the tail. The READ side takes
+// whatever misalignment that leaves it with: gfx950 global loads accept any address, and the
+// typedefs below tell the compiler so. Uneven shards therefore run the same unrolled code as
+// aligned ones; only head, tail and the last partial tile take guarded accesses.
+typedef u32x4 u32x4_u __attribute__((aligned(1)));
+typedef u32x2 u32x2_u __attribute__((aligned(1)));
+
+template <class V> struct Unaligned;
+template <> struct Unaligned<u32x4> { typedef u32x4_u type; };
+template <> struct Unaligned<u32x2> { typedef u32x2_u type; };
+
+template <class V>
+__device__ __forceinline__ V load_stream(const uint8_t* p) {  // nontemporal, any alignment
+  return __builtin_nontemporal_load(reinterpret_cast<const typename Unaligned<V>::type*>(p));
+}
+
+struct SegShape {
+  uint32_t head;   // units before the first vector boundary (clipped to the segment)
+  uint32_t tail;   // units after the last whole vector
+  uint64_t nvec;   // whole vectors
+  uint64_t last;   // tile that owns the tail
+};
+
+// unit_bytes: size of one unit; vec_units: units per vector (vec_units * unit_bytes is 8 or 16)
+__device__ __forceinline__ SegShape seg_shape(uintptr_t written_addr, uint64_t n, uint32_t unit_bytes,
+                                              uint32_t vec_units) {
+  const uint32_t vec_bytes = unit_bytes * vec_units;
+  SegShape g;
+  uint64_t head = ((vec_bytes - (uint32_t)(written_addr & (vec_bytes - 1))) & (vec_bytes - 1)) / unit_bytes;
+  if (head > n) head = n;
+  g.head = (uint32_t)head;
+  g.nvec = (n - head) / vec_units;
+  g.tail = (uint32_t)((n - head) - g.nvec * vec_units);
+  g.last = g.nvec ? (g.nvec - 1) / kTileVecs : 0;
+  return g;
 }
 
 // ---- gather -------------------------------------------------------------------------------
-// Copies n bytes d[0:n] = s[0:n] with the 256 threads of the block; any alignment. Stores are
-// 16 B aligned on the destination; the source side takes whatever misalignment is left.
-__device__ __forceinline__ void copy_any(uint8_t* d, const uint8_t* s, uint32_t n) {
+// Everything of a tile that is not a run of kTileVecs whole vectors: the last partial run, the
+// head and the tail. Kept out of line so that the streaming loop stays tight.
+__device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t* s, uint32_t chunk,
+                                                       SegShape g) {
   const uint32_t tid = threadIdx.x;
-  uint32_t head = (16u - (uint32_t)((uintptr_t)d & 15u)) & 15u;
-  if (head > n) head = n;
-  if (tid < head) d[tid] = s[tid];
-  d += head;
-  s += head;
-  n -= head;
-  const uint32_t nvec = n >> 4;
-  for (uint32_t v = tid; v < nvec; v += kThreads) {
-    const u32x4 x = load16_unaligned(s + (size_t)v * 16);
-    __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(d) + v);
+  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
+  if (v0 < g.nvec && v0 + kTileVecs > g.nvec) {
+    const uint32_t left = (uint32_t)(g.nvec - v0);
+    const uint8_t* sb = s + g.head + v0 * 16;
+    u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
+    u32x4 v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (u * kThreads + tid < left) v[u] = load_stream<u32x4>(sb + (size_t)(u * kThreads + tid) * 16);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (u * kThreads + tid < left) __builtin_nontemporal_store(v[u], db + u * kThreads + tid);
   }
-  const uint32_t tail = n & 15u;
-  if (tid < tail) d[(size_t)nvec * 16 + tid] = s[(size_t)nvec * 16 + tid];
+  if (chunk == 0 && tid < g.head) d[tid] = s[tid];
+  if (chunk == g.last && tid < g.tail) {
+    const uint64_t o = g.head + g.nvec * 16 + tid;
+    d[o] = s[o];
+  }
+}
+
+// True when tile `chunk` of a segment has anything besides whole runs of vectors to do.
+__device__ __forceinline__ bool has_edges(uint32_t chunk, const SegShape& g) {
+  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
+  return (v0 < g.nvec && v0 + kTileVecs > g.nvec) || (chunk == 0 && g.head) || (chunk == g.last && g.tail);
 }
 
 __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
+  const uint32_t tid = threadIdx.x;
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
     const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_bytes[c.item];
-    const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
-    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride +
-                       launch.src_off[c.item] + in_seg;
-    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg + in_seg;
-    const uint64_t left = seg - in_seg;
-    if (left >= kTileBytes && ((((uintptr_t)d) | ((uintptr_t)s)) & 15u) == 0) {
-      const u32x4* sv = reinterpret_cast<const u32x4*>(s) + threadIdx.x;
-      u32x4* dv = reinterpret_cast<u32x4*>(d) + threadIdx.x;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.src_off[c.item];
+    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg;
+    const SegShape g = seg_shape((uintptr_t)d, seg, 1, 16);
+    const uint64_t v0 = (uint64_t)c.chunk * kTileVecs;
+    if (v0 + kTileVecs <= g.nvec) {
+      const uint8_t* sb = s + g.head + (v0 + tid) * 16;
+      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0 + tid;
       u32x4 v[kUnroll];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(sv + u * kThreads);
+      for (int u = 0; u < kUnroll; ++u) v[u] = load_stream<u32x4>(sb + (size_t)u * kThreads * 16);
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], dv + u * kThreads);
-    } else {
-      copy_any(d, s, left < kTileBytes ? (uint32_t)left : kTileBytes);
+      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], db + u * kThreads);
     }
+    if (has_edges(c.chunk, g)) gather_edges(d, s, c.chunk, g);
   }
 }
 
 // ---- clear --------------------------------------------------------------------------------
-// Plain (not nontemporal) stores: for a write-only stream they measure ~3 % faster here.
+// Plain (not nontemporal) stores: for a write-only stream they measure faster here.
+__device__ __attribute__((noinline)) void clear_edges(uint8_t* d, uint32_t chunk, SegShape g) {
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const uint32_t tid = threadIdx.x;
+  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
+  if (v0 < g.nvec && v0 + kTileVecs > g.nvec) {
+    const uint32_t left = (uint32_t)(g.nvec - v0);
+    u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (u * kThreads + tid < left) db[u * kThreads + tid] = zero;
+  }
+  if (chunk == 0 && tid < g.head) d[tid] = 0;
+  if (chunk == g.last && tid < g.tail) d[g.head + g.nvec * 16 + tid] = 0;
+}
+
 __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launch) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
+  const uint32_t tid = threadIdx.x;
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
     const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_bytes[c.item];
-    const uint64_t in_seg = (uint64_t)c.chunk * kTileBytes;
-    uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.off[c.item] + in_seg;
-    const uint64_t left = seg - in_seg;
-    if (left >= kTileBytes && (((uintptr_t)d) & 15u) == 0) {
-      u32x4* dv = reinterpret_cast<u32x4*>(d) + threadIdx.x;
+    uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.off[c.item];
+    const SegShape g = seg_shape((uintptr_t)d, seg, 1, 16);
+    const uint64_t v0 = (uint64_t)c.chunk * kTileVecs;
+    if (v0 + kTileVecs <= g.nvec) {
+      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0 + tid;
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) dv[u * kThreads] = zero;
-    } else {
-      uint32_t n = left < kTileBytes ? (uint32_t)left : kTileBytes;
-      const uint32_t tid = threadIdx.x;
-      uint32_t head = (16u - (uint32_t)((uintptr_t)d & 15u)) & 15u;
-      if (head > n) head = n;
-      if (tid < head) d[tid] = 0;
-      d += head;
-      n -= head;
-      const uint32_t nvec = n >> 4;
-      for (uint32_t v = tid; v < nvec; v += kThreads)
-        reinterpret_cast<u32x4*>(d)[v] = zero;
-      const uint32_t tail = n & 15u;
-      if (tid < tail) d[(size_t)nvec * 16 + tid] = 0;
+      for (int u = 0; u < kUnroll; ++u) db[u * kThreads] = zero;
     }
+    if (has_edges(c.chunk, g)) clear_edges(d, c.chunk, g);
   }
 }
 
@@ -334,7 +386,7 @@ template <> struct Quad<f16_tag> {
 
 template <class G, class A>
 __device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uint64_t gi,
-                                          uint64_t grad_elems, uint32_t i) {
+                                          uint64_t grad_elems, uint64_t i) {
   typedef typename Codec<A>::raw_t araw_t;
   typedef typename Codec<G>::raw_t graw_t;
   araw_t* a = reinterpret_cast<araw_t*>(acc) + i;
@@ -343,64 +395,79 @@ __device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uin
   *a = Codec<A>::narrow(Codec<A>::widen(*a) + g);
 }
 
-// Slow path of one tile: acc[0:n] += grad[g0 : g0+n] (zero beyond grad_elems), any alignment.
+// One quad (4 elements) of a tile that is partial, crosses the end of the valid gradient, or
+// lies in the zero padding. acc points at the quad, gi is its first element's gradient index.
 template <class G, class A>
-__device__ __forceinline__ void accum_any(uint8_t* acc, const uint8_t* grad, uint64_t g0,
-                                          uint64_t grad_elems, uint32_t n) {
+__device__ __forceinline__ void accum_quad_guarded(uint8_t* acc, const uint8_t* grad, uint64_t gi,
+                                                   uint64_t grad_elems) {
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
-  constexpr uint32_t kAccVecBytes = 4 * Codec<A>::kBytes;
+  avec_t* ap = reinterpret_cast<avec_t*>(acc);
+  float gf[4] = {0.0f, 0.0f, 0.0f, 0.0f}, af[4];
+  if (gi + 4 <= grad_elems) {
+    Quad<G>::widen(load_stream<gvec_t>(grad + gi * Codec<G>::kBytes), gf);
+  } else {
+    typedef typename Codec<G>::raw_t graw_t;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (gi + k < grad_elems) gf[k] = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi + k]);
+  }
+  Quad<A>::widen(__builtin_nontemporal_load(ap), af);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
+  __builtin_nontemporal_store(Quad<A>::narrow(af), ap);
+}
+
+// The parts of a tile that are not whole runs of valid quads: a partial last run, a run that
+// crosses the end of the valid gradient or lies in the zero padding, the head and the tail.
+template <class G, class A>
+__device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_t* grad, uint64_t g_seg,
+                                                      uint64_t grad_elems, uint32_t chunk, SegShape g,
+                                                      bool body) {
+  constexpr uint32_t kAB = Codec<A>::kBytes;
   const uint32_t tid = threadIdx.x;
-  uint32_t head = ((kAccVecBytes - (uint32_t)((uintptr_t)acc & (kAccVecBytes - 1))) &
-                   (kAccVecBytes - 1)) / Codec<A>::kBytes;
-  if (head > n) head = n;
-  if (tid < head) accum_one<G, A>(acc, grad, g0 + tid, grad_elems, tid);
-  const uint32_t nvec = (n - head) >> 2;
-  for (uint32_t v = tid; v < nvec; v += kThreads) {
-    const uint32_t i = head + 4 * v;
-    const uint64_t gi = g0 + i;
-    if (gi + 4 <= grad_elems) {
-      gvec_t graw;
-      __builtin_memcpy(&graw, grad + gi * Codec<G>::kBytes, sizeof(gvec_t));
-      avec_t* ap = reinterpret_cast<avec_t*>(acc + (size_t)i * Codec<A>::kBytes);
-      float gf[4], af[4];
-      Quad<G>::widen(graw, gf);
-      Quad<A>::widen(*ap, af);
+  const uint64_t q0 = (uint64_t)chunk * kTileVecs;
+  if (body && q0 < g.nvec) {
+    const uint64_t left = g.nvec - q0;
+    const uint64_t e0 = g.head + q0 * 4;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
-      *ap = Quad<A>::narrow(af);
-    } else {
-#pragma unroll
-      for (int k = 0; k < 4; ++k) accum_one<G, A>(acc, grad, gi + k, grad_elems, i + k);
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t q = u * kThreads + tid;
+      if (q < left)
+        accum_quad_guarded<G, A>(acc + (e0 + (uint64_t)q * 4) * kAB, grad, g_seg + e0 + (uint64_t)q * 4, grad_elems);
     }
   }
-  const uint32_t done = head + 4 * nvec;
-  if (tid < n - done) accum_one<G, A>(acc, grad, g0 + done + tid, grad_elems, done + tid);
+  if (chunk == 0 && tid < g.head) accum_one<G, A>(acc, grad, g_seg + tid, grad_elems, tid);
+  if (chunk == g.last && tid < g.tail) {
+    const uint64_t i = g.head + g.nvec * 4 + tid;
+    accum_one<G, A>(acc, grad, g_seg + i, grad_elems, i);
+  }
 }
 
 template <class G, class A>
 __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launch) {
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
+  constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
+  const uint32_t tid = threadIdx.x;
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
     const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_elems[c.item];
-    const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
-    const uint64_t g0 = (uint64_t)c.rank * seg + in_seg;  // element index in the full gradient
     const uint64_t grad_elems = launch.grad_elems[c.item];
     const uint8_t* grad = launch.grad[c.item];
-    uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.acc_off[c.item] +
-                   in_seg * Codec<A>::kBytes;
-    const uint64_t left = seg - in_seg;
-    const uintptr_t gaddr = (uintptr_t)(grad + g0 * Codec<G>::kBytes);
-    if (left >= kTileElems && g0 + kTileElems <= grad_elems &&
-        (((uintptr_t)acc) & (sizeof(avec_t) - 1)) == 0 && (gaddr & (sizeof(gvec_t) - 1)) == 0) {
-      const gvec_t* gp = reinterpret_cast<const gvec_t*>(gaddr) + threadIdx.x;
-      avec_t* ap = reinterpret_cast<avec_t*>(acc) + threadIdx.x;
+    uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.acc_off[c.item];
+    const uint64_t g_seg = (uint64_t)c.rank * seg;  // gradient index of the segment's first element
+    const SegShape g = seg_shape((uintptr_t)acc, seg, kAB, 4);
+    const uint64_t q0 = (uint64_t)c.chunk * kTileVecs;  // first quad of this tile
+    const uint64_t e0 = g.head + q0 * 4;                // its first element within the segment
+    const bool whole = q0 + kTileVecs <= g.nvec && g_seg + e0 + kTileElems <= grad_elems;
+    if (whole) {
+      const uint8_t* gb = grad + (g_seg + e0) * kGB + (size_t)tid * sizeof(gvec_t);
+      avec_t* ap = reinterpret_cast<avec_t*>(acc + e0 * kAB) + tid;
       gvec_t graw[kUnroll];
       avec_t araw[kUnroll];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) graw[u] = __builtin_nontemporal_load(gp + u * kThreads);
+      for (int u = 0; u < kUnroll; ++u) graw[u] = load_stream<gvec_t>(gb + (size_t)u * kThreads * sizeof(gvec_t));
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) araw[u] = __builtin_nontemporal_load(ap + u * kThreads);
 #pragma unroll
@@ -412,9 +479,9 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
         for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
         __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * kThreads);
       }
-    } else {
-      accum_any<G, A>(acc, grad, g0, grad_elems, left < kTileElems ? (uint32_t)left : kTileElems);
     }
+    if (!whole || (c.chunk == 0 && g.head) || (c.chunk == g.last && g.tail))
+      accum_edges<G, A>(acc, grad, g_seg, grad_elems, c.chunk, g, !whole);
   }
 }
 
@@ -422,64 +489,66 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
 // dst[r*S + i] = narrow_D(widen_S(region_r[off + i])): the gather of shards kept in one dtype
 // (fp32 master copies) into a full parameter of another (bf16), in one pass.
 template <class S, class D>
-__device__ __forceinline__ void cast_one(uint8_t* d, const uint8_t* s, uint32_t i) {
+__device__ __forceinline__ void cast_one(uint8_t* d, const uint8_t* s, uint64_t i) {
   typedef typename Codec<S>::raw_t sraw_t;
   typedef typename Codec<D>::raw_t draw_t;
   reinterpret_cast<draw_t*>(d)[i] = Codec<D>::narrow(Codec<S>::widen(reinterpret_cast<const sraw_t*>(s)[i]));
 }
 
 template <class S, class D>
-__device__ __forceinline__ void cast_any(uint8_t* d, const uint8_t* s, uint32_t n) {
+__device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* s, uint32_t chunk, SegShape g) {
   typedef typename Quad<S>::vec_t svec_t;
   typedef typename Quad<D>::vec_t dvec_t;
-  constexpr uint32_t kDstVecBytes = 4 * Codec<D>::kBytes;
+  constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
   const uint32_t tid = threadIdx.x;
-  uint32_t head = ((kDstVecBytes - (uint32_t)((uintptr_t)d & (kDstVecBytes - 1))) &
-                   (kDstVecBytes - 1)) / Codec<D>::kBytes;
-  if (head > n) head = n;
-  if (tid < head) cast_one<S, D>(d, s, tid);
-  const uint32_t nvec = (n - head) >> 2;
-  for (uint32_t v = tid; v < nvec; v += kThreads) {
-    const uint32_t i = head + 4 * v;
-    svec_t raw;
-    __builtin_memcpy(&raw, s + (size_t)i * Codec<S>::kBytes, sizeof(svec_t));
-    float f[4];
-    Quad<S>::widen(raw, f);
-    __builtin_nontemporal_store(Quad<D>::narrow(f),
-                                reinterpret_cast<dvec_t*>(d + (size_t)i * Codec<D>::kBytes));
+  const uint64_t q0 = (uint64_t)chunk * kTileVecs;
+  if (q0 < g.nvec && q0 + kTileVecs > g.nvec) {
+    const uint64_t left = g.nvec - q0;
+    const uint64_t e0 = g.head + q0 * 4;
+    const uint8_t* sb = s + e0 * kSB;
+    dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t q = u * kThreads + tid;
+      if (q < left) {
+        float f[4];
+        Quad<S>::widen(load_stream<svec_t>(sb + (size_t)q * sizeof(svec_t)), f);
+        __builtin_nontemporal_store(Quad<D>::narrow(f), dp + q);
+      }
+    }
   }
-  const uint32_t done = head + 4 * nvec;
-  if (tid < n - done) cast_one<S, D>(d, s, done + tid);
+  if (chunk == 0 && tid < g.head) cast_one<S, D>(d, s, tid);
+  if (chunk == g.last && tid < g.tail) cast_one<S, D>(d, s, g.head + g.nvec * 4 + tid);
 }
 
 template <class S, class D>
 __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherLaunch launch) {
   typedef typename Quad<S>::vec_t svec_t;
   typedef typename Quad<D>::vec_t dvec_t;
+  constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
+  const uint32_t tid = threadIdx.x;
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
     const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_elems[c.item];
-    const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
-    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride +
-                       launch.src_off[c.item] + in_seg * Codec<S>::kBytes;
-    uint8_t* d = launch.dst[c.item] + ((uint64_t)c.rank * seg + in_seg) * Codec<D>::kBytes;
-    const uint64_t left = seg - in_seg;
-    if (left >= kTileElems && (((uintptr_t)s) & (sizeof(svec_t) - 1)) == 0 &&
-        (((uintptr_t)d) & (sizeof(dvec_t) - 1)) == 0) {
-      const svec_t* sp = reinterpret_cast<const svec_t*>(s) + threadIdx.x;
-      dvec_t* dp = reinterpret_cast<dvec_t*>(d) + threadIdx.x;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.src_off[c.item];
+    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg * kDB;
+    const SegShape g = seg_shape((uintptr_t)d, seg, kDB, 4);
+    const uint64_t q0 = (uint64_t)c.chunk * kTileVecs;
+    if (q0 + kTileVecs <= g.nvec) {
+      const uint64_t e0 = g.head + q0 * 4;
+      const uint8_t* sb = s + e0 * kSB + (size_t)tid * sizeof(svec_t);
+      dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB) + tid;
       svec_t raw[kUnroll];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) raw[u] = __builtin_nontemporal_load(sp + u * kThreads);
+      for (int u = 0; u < kUnroll; ++u) raw[u] = load_stream<svec_t>(sb + (size_t)u * kThreads * sizeof(svec_t));
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         float f[4];
         Quad<S>::widen(raw[u], f);
         __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * kThreads);
       }
-    } else {
-      cast_any<S, D>(d, s, left < kTileElems ? (uint32_t)left : kTileElems);
     }
+    if (has_edges(c.chunk, g)) cast_edges<S, D>(d, s, c.chunk, g);
   }
 }
 
