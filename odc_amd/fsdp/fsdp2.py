@@ -18,6 +18,15 @@ copies out per parameter (and, the other way, ``chunk_cat``s gradients into ``[W
 before the scatter-accumulate); ``fused=True`` (default) lets the kernels' work lists do both
 directly, ``fused=False`` keeps the reference's two-step data flow.
 
+The same data flow is wired into torch's own ``fully_shard`` modules by ``patch_fsdp2`` +
+``patch_lazy_init`` (fsdp2.py:103-112, 1105-1138): torch's ``foreach_all_gather``,
+``foreach_all_gather_copy_out`` and ``foreach_reduce`` are replaced with versions that gather the
+group's symmetric buffer straight into the parameters' unsharded storage (dtype conversion fused)
+and scatter-accumulate the unsharded gradients straight into the group's accumulation; gradients
+are handed to the sharded parameters at ``pre_optimizer_step``. One process plays one rank of a W
+rank mesh (for instance over torch's "fake" process-group backend); the other ranks' shards are
+passive memory, filled with ``fill_peer_shards``.
+
 HPZ (fsdp2.py:551-582, 745-791, 961-1099) and the HSDP all-reduce (fsdp2.py:849-885) need more
 than one node and are not part of this build.
 """
@@ -202,13 +211,269 @@ class ParamGroup:
         return grads
 
 
+# ------------------------------------------------------------------------------------------------
+# torch fully_shard integration
+# ------------------------------------------------------------------------------------------------
+def _torch_param_groups(fsdp_module):
+    """All FSDPParamGroups under a ``fully_shard`` root module (fsdp2.py:1026-1030)."""
+    from torch.distributed.fsdp import fully_shard
+
+    root_state = fully_shard.state(fsdp_module)
+    root_state._lazy_init()
+    return [
+        st._fsdp_param_group for st in root_state._state_ctx.all_states if st._fsdp_param_group is not None
+    ]
+
+
+def _group_layout(fsdp_param_group):
+    return fsdp_param_group._odc_layout
+
+
+class _GroupLayout:
+    """Where each FSDPParam of a torch param group lives in the group's symmetric buffer."""
+
+    def __init__(self, fsdp_param_group):
+        params = fsdp_param_group.fsdp_params
+        self.key = get_fsdp_params_key([id(p) for p in params])
+        self.dtype = params[0]._sharded_param_data.dtype
+        for fp in params:
+            if fp._sharded_param_data.dtype != self.dtype:
+                raise ValueError(
+                    f"All FSDP parameters must have the same dtype: {fp._sharded_param_data.dtype=} {self.dtype=}"
+                )
+            if fp.fsdp_placement.dim != 0:
+                raise NotImplementedError("only dim-0 sharding is wired to the fused kernels")
+        self.numels = [fp._sharded_param_data.numel() for fp in params]
+        self.offsets = [0]
+        for n in self.numels:
+            self.offsets.append(self.offsets[-1] + n)
+        self.total = self.offsets.pop()
+        self.index = {id(fp): i for i, fp in enumerate(params)}
+
+
+@torch.no_grad()
+def replace_sharded_param_with_symm_buffer(fsdp_model) -> None:
+    """Move the group's sharded parameters into one symmetric buffer and point the FSDPParams
+    (and their DTensors' local tensors) at views of it (fsdp2.py:116-202, without HPZ)."""
+    if _enable_hpz is None:
+        raise ValueError("Need to run patch_fsdp2() first")
+    group = fsdp_model._get_fsdp_state()._fsdp_param_group
+    if group is None or hasattr(group, "_odc_layout"):
+        return
+    layout = _GroupLayout(group)
+    symm_buffer = SymmBufferRegistry.get_instance().get_or_create_symm_buffer(
+        layout.key, (layout.total,), layout.dtype
+    )
+    for fp, off, n in zip(group.fsdp_params, layout.offsets, layout.numels):
+        assert math.prod(fp.padded_sharded_param_size) == n
+        piece = symm_buffer[off : off + n]
+        piece.copy_(fp._sharded_param_data)
+        padded = piece.view(fp.padded_sharded_param_size)
+        fp._sharded_param_data = padded.view(-1)
+        old_local = fp.sharded_param._local_tensor
+        length = old_local.size(0) if old_local.numel() > 0 else 0
+        fp.sharded_param._local_tensor = padded.narrow(dim=0, start=0, length=length)
+        fp._odc_group = group
+    group._odc_layout = layout
+    group._odc_symm_buffer = symm_buffer
+
+
+@torch.no_grad()
+def patch_lazy_init(fsdp_model) -> None:
+    """Run ``replace_sharded_param_with_symm_buffer`` right after the group's own lazy init
+    (fsdp2.py:103-112)."""
+    import types
+
+    group = fsdp_model._get_fsdp_state()._fsdp_param_group
+    if group is None:
+        return
+    prev_lazy_init = group.lazy_init
+
+    def patched_lazy_init(_self):
+        prev_lazy_init()
+        replace_sharded_param_with_symm_buffer(fsdp_model)
+
+    group.lazy_init = types.MethodType(patched_lazy_init, group)
+
+
+@torch.no_grad()
+def fill_peer_shards(fsdp_model, full_params) -> None:
+    """Virtual-world helper: write rank r's chunk of every full parameter into rank r's region,
+    for all r (in the reference every process does this for itself at lazy init).
+    ``full_params`` maps a parameter's fully qualified name (as the root module names it) to
+    the full, unsharded tensor."""
+    group = fsdp_model._get_fsdp_state()._fsdp_param_group
+    if group is None:
+        return
+    layout = _group_layout(group)
+    peers = SymmBufferRegistry.get_instance().peer_tensors[layout.key]
+    W = len(peers)
+    for fp, off, n in zip(group.fsdp_params, layout.offsets, layout.numels):
+        full = full_params[fp._param_fqn]
+        rows = math.ceil(full.shape[0] / W)
+        for r in range(W):
+            chunk = full[r * rows : (r + 1) * rows].reshape(-1).to(layout.dtype)
+            peers[r][off : off + n].zero_()
+            peers[r][off : off + chunk.numel()].copy_(chunk)
+
+
+@torch.no_grad()
+def foreach_all_gather(fsdp_params, group, async_op, all_gather_copy_in_stream, all_gather_stream,
+                       device, all_gather_comm):
+    """Replacement for torch's ``foreach_all_gather`` (fsdp2.py:219-313): no copy-in, no
+    intermediate ``[W, sum n_p]`` buffer — the group's symmetric buffer is gathered straight into
+    every parameter's unsharded storage, converted to ``param_dtype`` on the way."""
+    from torch.distributed.device_mesh import _get_device_handle
+    from torch.distributed.fsdp._fully_shard._fsdp_collectives import AllGatherResult
+
+    fsdp_group = fsdp_params[0]._odc_group
+    layout = _group_layout(fsdp_group)
+    world_size = group.size()
+    device_handle = _get_device_handle(device.type)
+    out_dtype = fsdp_params[0].param_dtype or layout.dtype
+    outs, offsets, numels, dtypes_meta, numels_meta = [], [], [], [], []
+    for fp in fsdp_params:
+        i = layout.index[id(fp)]
+        n = layout.numels[i]
+        fp.init_all_gather_outputs([n], [out_dtype], world_size, device)
+        fp.alloc_all_gather_outputs()  # on the current stream, where torch allocates them too
+        outs.append(fp.all_gather_outputs[0])
+        offsets.append(layout.offsets[i])
+        numels.append(n)
+        dtypes_meta.append([out_dtype])
+        numels_meta.append([n])
+    all_gather_stream.wait_stream(all_gather_copy_in_stream)
+    with device_handle.stream(all_gather_stream):
+        get_gather_service().gather_slices(outs, fsdp_group._odc_symm_buffer, offsets, numels, group)
+        all_gather_event = all_gather_stream.record_event()
+    placeholder = torch.empty(0, dtype=out_dtype, device=device)
+    return AllGatherResult(placeholder, all_gather_event, None, dtypes_meta, numels_meta, numels)
+
+
+@torch.no_grad()
+def foreach_all_gather_copy_out(all_gather_result, fsdp_params, group) -> None:
+    """The copy-out already happened inside the gather; only the stream dependency is left
+    (fsdp2.py:317-424)."""
+    event = all_gather_result.all_gather_event
+    if event is not None:
+        torch.cuda.current_stream().wait_event(event)
+
+
+@torch.no_grad()
+def foreach_reduce(fsdp_params, unsharded_grads, reduce_scatter_group, reduce_scatter_stream,
+                   reduce_scatter_comm, orig_dtype, reduce_dtype, device, gradient_divide_factor,
+                   all_reduce_group, all_reduce_stream, all_reduce_grads, partial_reduce_output,
+                   all_reduce_hook, force_sum_reduction_for_comms=False):
+    """Replacement for torch's ``foreach_reduce`` (fsdp2.py:608-742): the unsharded gradients are
+    scatter-accumulated straight into the group's accumulation (zero padding and the cast to the
+    reduce dtype happen in the kernel); handing gradients to the sharded parameters is deferred
+    to ``pre_optimizer_step``."""
+    from torch.distributed.device_mesh import _get_device_handle
+    from torch.distributed.fsdp._fully_shard._fsdp_collectives import (
+        _div_if_needed,
+        _get_gradient_divide_factors,
+    )
+
+    if all_reduce_group is not None:
+        raise NotImplementedError("HSDP needs more than one node; not part of this build")
+    grad_dtypes = {g.dtype for g in unsharded_grads}
+    if len(grad_dtypes) != 1:
+        raise AssertionError(f"FSDP reduce-scatter expects uniform gradient dtype but got {grad_dtypes}")
+    grad_dtype = unsharded_grads[0].dtype
+    reduce_dtype = reduce_dtype or grad_dtype
+    predivide_factor, _post, _rs_op, _ar_op = _get_gradient_divide_factors(
+        reduce_scatter_group, all_reduce_group, reduce_dtype, device.type, gradient_divide_factor,
+        force_sum_reduction_for_comms,
+    )
+    fsdp_group = fsdp_params[0]._odc_group
+    layout = _group_layout(fsdp_group)
+    device_handle = _get_device_handle(device.type)
+    current_stream = device_handle.current_stream()
+    reduce_scatter_stream.wait_stream(current_stream)
+    with device_handle.stream(reduce_scatter_stream):
+        grads, offsets, numels = [], [], []
+        for fp, g in zip(fsdp_params, unsharded_grads):
+            i = layout.index[id(fp)]
+            g = g.contiguous().view(-1)
+            _div_if_needed(g, predivide_factor)
+            g.record_stream(reduce_scatter_stream)  # read there after the caller drops its list
+            grads.append(g)
+            offsets.append(layout.offsets[i])
+            numels.append(layout.numels[i])
+        get_reduction_service().scatter_accumulate_slices(
+            id(fsdp_group), grads, offsets, numels, reduce_scatter_group,
+            accumulation_numel=layout.total, accumulation_dtype=reduce_dtype,
+        )
+        reduce_scatter_event = reduce_scatter_stream.record_event()
+        fsdp_group._odc_reduce_context = dict(
+            reduce_scatter_group=reduce_scatter_group, reduce_scatter_stream=reduce_scatter_stream,
+            orig_dtype=orig_dtype, reduce_dtype=reduce_dtype, device=device,
+            gradient_divide_factor=gradient_divide_factor, all_reduce_hook=all_reduce_hook,
+            force_sum_reduction_for_comms=force_sum_reduction_for_comms, grad_dtype=grad_dtype,
+        )
+        post_reduce_event = reduce_scatter_stream.record_event()
+    unsharded_grads.clear()
+    placeholder = torch.empty(0, dtype=reduce_dtype, device=device)
+    return placeholder, reduce_scatter_event, post_reduce_event, None, None, partial_reduce_output
+
+
+@torch.no_grad()
+def update_gradients(fsdp_param_group) -> None:
+    """fsdp2.py:795-957 for a torch param group: average and post-divide the calling rank's
+    accumulation in place, cast to the parameter dtype, hand the strided views to the sharded
+    parameters as DTensor gradients."""
+    import torch.distributed as dist
+    from torch.distributed.fsdp._fully_shard._fsdp_collectives import _get_gradient_divide_factors
+    from torch.distributed.tensor import DTensor
+
+    ctx = getattr(fsdp_param_group, "_odc_reduce_context", None)
+    if ctx is None:
+        return  # no microbatch ran through this group in this minibatch (fsdp2.py:797-801)
+    del fsdp_param_group._odc_reduce_context
+    layout = _group_layout(fsdp_param_group)
+    rs_group = ctx["reduce_scatter_group"]
+    _pre, postdivide_factor, reduce_scatter_op, _ar_op = _get_gradient_divide_factors(
+        rs_group, None, ctx["reduce_dtype"], ctx["device"].type, ctx["gradient_divide_factor"],
+        ctx["force_sum_reduction_for_comms"],
+    )
+    assert reduce_scatter_op in (dist.ReduceOp.SUM, dist.ReduceOp.AVG), f"{reduce_scatter_op} is not supported"
+    scatter = get_reduction_service()
+    key = id(fsdp_param_group)
+    orig_dtype = ctx["orig_dtype"] or scatter.get_accumulation(key).dtype
+    if ctx["all_reduce_hook"] is not None or (postdivide_factor is not None and postdivide_factor > 1):
+        # two roundings (average, then post-divide) and a user hook in between
+        if reduce_scatter_op == dist.ReduceOp.AVG:
+            scatter.publish([key], divisor=float(rs_group.size()))
+        if ctx["all_reduce_hook"] is not None:
+            ctx["all_reduce_hook"](scatter.get_accumulation(key))
+        divisor = postdivide_factor if postdivide_factor is not None and postdivide_factor > 1 else 1.0
+        (reduce_output,) = scatter.publish([key], out_dtype=orig_dtype, divisor=divisor)
+    else:
+        divisor = float(rs_group.size()) if reduce_scatter_op == dist.ReduceOp.AVG else 1.0
+        (reduce_output,) = scatter.publish([key], out_dtype=orig_dtype, divisor=divisor)
+    base = reduce_output.storage_offset()
+    for fp, off in zip(fsdp_param_group.fsdp_params, layout.offsets):
+        new_sharded_grad = torch.as_strided(
+            reduce_output, size=fp.sharded_size, stride=fp.contiguous_sharded_stride,
+            storage_offset=base + off,
+        )
+        if fp.sharded_param.grad is not None:
+            assert isinstance(fp.sharded_param.grad, DTensor)
+            fp.sharded_param.grad._local_tensor += new_sharded_grad
+        else:
+            fp.sharded_param.grad = fp.to_sharded_dtensor(new_sharded_grad)
+        for hook in (getattr(fp.sharded_param, "_post_accumulate_grad_hooks", {}) or {}).values():
+            hook(fp.sharded_param)
+
+
+def _is_torch_fsdp_module(fsdp_module) -> bool:
+    return hasattr(fsdp_module, "_get_fsdp_state")
+
+
 def _param_groups(fsdp_module) -> List[ParamGroup]:
     groups = getattr(fsdp_module, "_odc_param_groups", None)
     if groups is None:
-        raise NotImplementedError(
-            "expected an object with `_odc_param_groups` (a list of ParamGroup); rewiring a real "
-            "torch fully_shard module needs a process group of W real ranks and is not done here"
-        )
+        raise TypeError("expected a fully_shard module or an object with `_odc_param_groups`")
     return list(groups)
 
 
@@ -222,6 +487,14 @@ def pre_minibatch_start(fsdp_module):
 def pre_optimizer_step(fsdp_module):
     """fsdp2.py:1023-1046: sync once, then publish every group's gradients."""
     scatter = get_reduction_service()
+    if _is_torch_fsdp_module(fsdp_module):
+        for i, group in enumerate(_torch_param_groups(fsdp_module)):
+            if i == 0:
+                with torch.cuda.nvtx.range("scatter_accumulate_sync"):
+                    scatter.sync(group.mesh_info.shard_process_group)
+            with torch.cuda.nvtx.range(f"update_gradients:{group._module_fqn}"):
+                update_gradients(group)
+        return
     for i, group in enumerate(_param_groups(fsdp_module)):
         if i == 0:
             with torch.cuda.nvtx.range("scatter_accumulate_sync"):
@@ -231,13 +504,35 @@ def pre_optimizer_step(fsdp_module):
 
 
 def patch_fsdp2(enable_hpz: bool = False) -> None:
-    """Create the two services (fsdp2.py:1135-1138)."""
+    """Create the two services and route torch's fully_shard collectives through them
+    (fsdp2.py:1105-1138). Modules sharded afterwards need ``patch_lazy_init(module)`` each."""
     global _enable_hpz, reduction_service, gather_service
     if enable_hpz:
         raise NotImplementedError("HPZ needs more than one node; not part of this build")
     _enable_hpz = False
+    from torch.distributed.fsdp._fully_shard import _fsdp_collectives, _fsdp_param_group
+
+    for module in (_fsdp_collectives, _fsdp_param_group):
+        if not hasattr(module, "_odc_original_collectives"):
+            module._odc_original_collectives = (
+                module.foreach_all_gather, module.foreach_all_gather_copy_out, module.foreach_reduce,
+            )
+        module.foreach_all_gather = foreach_all_gather
+        module.foreach_all_gather_copy_out = foreach_all_gather_copy_out
+        module.foreach_reduce = foreach_reduce
     reduction_service = ReductionService()
     gather_service = GatherService()
+
+
+def unpatch_fsdp2() -> None:
+    """Put torch's own collectives back (for running patched and unpatched in one process)."""
+    from torch.distributed.fsdp._fully_shard import _fsdp_collectives, _fsdp_param_group
+
+    for module in (_fsdp_collectives, _fsdp_param_group):
+        orig = getattr(module, "_odc_original_collectives", None)
+        if orig is not None:
+            module.foreach_all_gather, module.foreach_all_gather_copy_out, module.foreach_reduce = orig
+            del module._odc_original_collectives
 
 
 def stop():

@@ -1,0 +1,141 @@
+"""torch's own fully_shard (FSDP2) trained through the primitives: one process plays rank 0 of a
+W-rank mesh over torch's "fake" process-group backend; the other ranks' shards are passive memory
+in the symmetric arena. Checked against the same model run unsharded."""
+
+import copy
+import math
+
+import pytest
+import torch
+import torch.distributed as dist
+import torch.nn as nn
+
+from helpers import assert_bit_equal
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+class Block(nn.Module):
+    def __init__(self, dim, hidden):
+        super().__init__()
+        self.norm = nn.LayerNorm(dim)
+        self.up = nn.Linear(dim, hidden)
+        self.down = nn.Linear(hidden, dim, bias=False)
+
+    def forward(self, x):
+        return x + self.down(torch.relu(self.up(self.norm(x))))
+
+
+class Toy(nn.Module):
+    def __init__(self, dim=96, hidden=50, layers=3, out=10):
+        super().__init__()
+        self.inp = nn.Linear(32, dim)
+        self.layers = nn.ModuleList([Block(dim, hidden) for _ in range(layers)])
+        self.head = nn.Linear(dim, out)
+
+    def forward(self, x):
+        x = self.inp(x)
+        for layer in self.layers:
+            x = layer(x)
+        return self.head(x)
+
+
+@pytest.fixture
+def fake_process_group():
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    def _init(world_size):
+        dist.init_process_group("fake", rank=0, world_size=world_size, store=FakeStore())
+
+    yield _init
+    from odc_amd.fsdp import fsdp2
+
+    fsdp2.unpatch_fsdp2()
+    if dist.is_initialized():
+        dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("W", [4, 8])
+@pytest.mark.parametrize("mixed", [True, False])
+def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_group, W, mixed):
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.fsdp import MixedPrecisionPolicy, fully_shard
+
+    from odc_amd.fsdp import fsdp2
+
+    fake_process_group(W)
+    mesh = init_device_mesh("cuda", (W,))
+    make_world(W, 64 << 20)
+    fsdp2.patch_fsdp2()
+
+    torch.manual_seed(0)
+    model = Toy().cuda()
+    reference = copy.deepcopy(model)
+    full_params = {name: p.detach().clone() for name, p in reference.named_parameters()}
+    kwargs = {"mesh": mesh}
+    if mixed:
+        kwargs["mp_policy"] = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
+    for layer in model.layers:
+        fully_shard(layer, **kwargs)
+    fully_shard(model, **kwargs)
+    for layer in model.layers:
+        fsdp2.patch_lazy_init(layer)
+    fsdp2.patch_lazy_init(model)
+    fully_shard.state(model)._lazy_init()  # moves the shards into the symmetric arena
+    for module in [*model.layers, model]:
+        fsdp2.fill_peer_shards(module, full_params)
+    breakdown = fsdp2.get_symm_buffer_memory_breakdown()
+    assert set(breakdown) >= {"fsdp_params", "accumulation"}
+    # rank 0's shard of every parameter is chunk 0 of the full parameter, living in the arena
+    for name, p in model.named_parameters():
+        local = p._local_tensor
+        rows = math.ceil(full_params[name].shape[0] / W)
+        assert_bit_equal(local, full_params[name][:rows], f"local shard of {name}")
+        arena = __import__("odc_amd").primitives.utils.get_world().arena
+        assert arena.locate(local.data_ptr())[0] == 0  # it lives in rank 0's region of the arena
+
+    compute_dtype = torch.bfloat16 if mixed else torch.float32
+    ref_compute = copy.deepcopy(reference).to(compute_dtype)
+    M = 3
+    g = torch.Generator().manual_seed(1)
+    batches = [torch.randn(16, 32, generator=g).cuda() for _ in range(M)]
+
+    fsdp2.pre_minibatch_start(model)
+    want = {name: torch.zeros(p.numel()) for name, p in full_params.items()}
+    for x in batches:
+        model(x).float().pow(2).mean().backward()
+        ref_compute.zero_grad(set_to_none=True)
+        ref_compute(x.to(compute_dtype)).float().pow(2).mean().backward()
+        for name, p in ref_compute.named_parameters():
+            want[name].add_(p.grad.detach().cpu().reshape(-1))  # fp32 += compute-dtype grad, in order
+    fsdp2.pre_optimizer_step(model)
+
+    for name, p in model.named_parameters():
+        rows = math.ceil(full_params[name].shape[0] / W)
+        local_rows = min(rows, full_params[name].shape[0])
+        rest = full_params[name][0].numel() if full_params[name].dim() > 1 else 1
+        expect = oracle.fsdp2_average(want[name][: local_rows * rest].clone(), W).view(p._local_tensor.shape)
+        got = p.grad._local_tensor
+        assert got.dtype == torch.float32 and got.shape == expect.shape
+        assert_bit_equal(got, expect, f"sharded gradient of {name}")
+
+    # the optimizer updates rank 0's shards in place, i.e. inside the arena; the next gather sees them
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    before = {name: p._local_tensor.clone() for name, p in model.named_parameters()}
+    opt.step()
+    for name, p in model.named_parameters():
+        assert_bit_equal(
+            p._local_tensor, torch.add(before[name], p.grad._local_tensor, alpha=-0.1), f"updated shard of {name}"
+        )
+    updated = {name: p._local_tensor.clone() for name, p in model.named_parameters()}
+    opt.zero_grad()
+    fsdp2.pre_minibatch_start(model)
+    out = model(batches[0])
+    # reference with chunk 0 of every parameter updated and the other chunks unchanged
+    with torch.no_grad():
+        for name, p in reference.named_parameters():
+            rows = math.ceil(p.shape[0] / W)
+            p[:rows] = updated[name]
+    want_out = copy.deepcopy(reference).to(compute_dtype)(batches[0].to(compute_dtype))
+    assert_bit_equal(out, want_out, "forward after the optimizer step")
