@@ -11,7 +11,9 @@ primitives, provided here as plain functions with the same meaning:
 plus ``pre_minibatch_start`` / ``pre_optimizer_step`` / ``stop`` / ``patch_fsdp1`` with the
 reference's signatures. The hooks take any object with the attributes the reference reads from
 torch's ``_FSDPState`` (``process_group``, ``_gradient_postdivide_factor``, ``_all_handles`` whose
-items carry ``flat_param``), so they also serve stand-in modules.
+items carry ``flat_param``), so they also serve stand-in modules. ``patch_fsdp1`` installs the call
+sites into torch's ``FullyShardedDataParallel``; one process then plays one rank of a W-rank
+process group (for instance torch's "fake" backend).
 """
 
 from __future__ import annotations
@@ -101,13 +103,122 @@ def reduce_grad(flat_param, unsharded_grad: torch.Tensor, pg, predivide_factor: 
     return service.get_accumulation(key)
 
 
+# ------------------------------------------------------------------------------------------------
+# torch FullyShardedDataParallel integration (the monkey patches of fsdp1.py:302-314)
+# ------------------------------------------------------------------------------------------------
+_originals = {}
+
+
+def _patched_get_shard(tensor, rank, world_size):
+    """``FlatParamHandle._get_shard`` (fsdp1.py:239-247): the calling rank's padded chunk, living
+    in its symmetric buffer. One process holds all W virtual ranks, so every rank's chunk is
+    published here (in the reference each process publishes its own)."""
+    from torch.distributed.fsdp._flat_param import FlatParameter
+
+    assert isinstance(tensor, FlatParameter)
+    registry = odc_amd.SymmBufferRegistry.get_instance()
+    original = _originals["_get_shard"]
+    local, local_pad = None, 0
+    for r in range(world_size):
+        sharded, numel_to_pad = original(tensor, r, world_size)
+        with odc_amd.virtual_rank(r):
+            in_symm = registry.update_symm_buffer(id(tensor), sharded)
+        if r == rank:
+            local, local_pad = in_symm, numel_to_pad
+    return local, local_pad
+
+
+def _patched_all_gather_flat_param(self, padded_unsharded_flat_param):
+    """``FlatParamHandle._all_gather_flat_param`` (fsdp1.py:156-233)."""
+    sharded_flat_param = self.flat_param.data
+    pg = self._fake_process_group if self._use_fake_all_gather else self.process_group
+    assert not sharded_flat_param.is_cpu and not self._offload_params, "ODC does not support offloading"
+    return all_gather_flat_param(
+        padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=self._fwd_bwd_param_dtype
+    )
+
+
+def _patched_use_low_precision_shard(self):
+    """No low-precision copy of the shard is made: peers read the shard in its own dtype and
+    the gather converts (fsdp1.py:250-275)."""
+    self._check_low_precision_shard()
+
+
+def _patched_free_low_precision_sharded_param(self):
+    self._check_low_precision_shard()  # nothing was allocated (fsdp1.py:278-299)
+
+
+def _patched_reduce_grad(state, handle) -> None:
+    """``_runtime_utils._reduce_grad`` (fsdp1.py:41-106)."""
+    from torch.distributed.fsdp._flat_param import HandleShardingStrategy
+
+    flat_param = handle.flat_param
+    assert handle._sharding_strategy not in (
+        HandleShardingStrategy.HYBRID_SHARD,
+        HandleShardingStrategy._HYBRID_SHARD_ZERO2,
+    ), "ODC does not support hybrid sharded strategy"
+    assert state._comm_hook is None, "ODC does not support comm hook"
+    assert not handle._offload_params, "ODC does not support offloading"
+    assert not handle._use_orig_params, "ODC does not support using original parameters"
+    unsharded_grad = flat_param.grad.data
+    flat_param.grad = None  # permits several backwards per minibatch
+    pg = handle._fake_process_group if handle._use_fake_reduce else state.process_group
+    flat_param._saved_grad_shard = reduce_grad(
+        flat_param, unsharded_grad, pg, predivide_factor=state._gradient_predivide_factor
+    )
+
+
+def _patched_prepare_gradient_for_optim(self):
+    """``FlatParamHandle.prepare_gradient_for_optim`` (fsdp1.py:109-153): at the end of a backward
+    the accumulation is NOT forwarded to ``.grad``; ``pre_optimizer_step`` publishes it."""
+    flat_param = self.flat_param
+    assert not hasattr(flat_param, "_cpu_grad"), "ODC does not support offloading"
+    if hasattr(flat_param, "_saved_grad_shard"):
+        self._check_sharded(flat_param)
+        if flat_param._post_backward_called:
+            flat_param.grad = None
+        delattr(flat_param, "_saved_grad_shard")
+
+
 def patch_fsdp1(reduce_dtype=None):
-    """Create the two services (fsdp1.py:302-305). Rewiring torch's FlatParamHandle to call
-    ``get_shard`` / ``all_gather_flat_param`` / ``reduce_grad`` needs a process group of W real
-    ranks and is not done here."""
+    """Create the two services and route torch FSDP1's all-gather and reduce-scatter through
+    them (fsdp1.py:302-314). Call before wrapping modules: shards move into the symmetric arena
+    when ``FullyShardedDataParallel`` shards its flat parameters."""
     global reduction_service, gather_service
     reduction_service = odc_amd.ReductionService(accumulation_dtype=reduce_dtype)
     gather_service = odc_amd.GatherService()
+    from torch.distributed.fsdp import _runtime_utils
+    from torch.distributed.fsdp._flat_param import FlatParamHandle
+
+    if not _originals:
+        _originals.update(
+            _reduce_grad=_runtime_utils._reduce_grad,
+            prepare_gradient_for_optim=FlatParamHandle.prepare_gradient_for_optim,
+            _get_shard=FlatParamHandle._get_shard,
+            _all_gather_flat_param=FlatParamHandle._all_gather_flat_param,
+            _use_low_precision_shard=FlatParamHandle._use_low_precision_shard,
+            _free_low_precision_sharded_param=FlatParamHandle._free_low_precision_sharded_param,
+        )
+    _runtime_utils._reduce_grad = _patched_reduce_grad
+    FlatParamHandle.prepare_gradient_for_optim = _patched_prepare_gradient_for_optim
+    FlatParamHandle._get_shard = staticmethod(_patched_get_shard)
+    FlatParamHandle._all_gather_flat_param = _patched_all_gather_flat_param
+    FlatParamHandle._use_low_precision_shard = _patched_use_low_precision_shard
+    FlatParamHandle._free_low_precision_sharded_param = _patched_free_low_precision_sharded_param
+
+
+def unpatch_fsdp1():
+    """Put torch's own methods back (for running patched and unpatched in one process)."""
+    if not _originals:
+        return
+    from torch.distributed.fsdp import _runtime_utils
+    from torch.distributed.fsdp._flat_param import FlatParamHandle
+
+    _runtime_utils._reduce_grad = _originals.pop("_reduce_grad")
+    FlatParamHandle._get_shard = staticmethod(_originals.pop("_get_shard"))
+    for name, fn in list(_originals.items()):
+        setattr(FlatParamHandle, name, fn)
+    _originals.clear()
 
 
 def pre_optimizer_step(fsdp_module):

@@ -30,6 +30,10 @@ def make_world():
         return group
 
     yield _make
+    from odc_amd.fsdp import fsdp1, fsdp2
+
+    fsdp1.unpatch_fsdp1()
+    fsdp2.unpatch_fsdp2()
     if utils.is_initialized():
         torch.cuda.synchronize()
         utils.SymmBufferRegistry.get_instance().finalize()

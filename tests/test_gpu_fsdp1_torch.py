@@ -1,0 +1,116 @@
+"""torch's FullyShardedDataParallel (FSDP1) trained through the primitives: one process plays rank 0
+of a W-rank group over torch's "fake" process-group backend; all W flat-parameter shards live in the
+symmetric arena. Checked against the same model run unsharded, with the oracle doing the
+accumulation arithmetic."""
+
+import copy
+import math
+
+import pytest
+import torch
+import torch.distributed as dist
+
+from helpers import assert_bit_equal
+from oracle import odc_oracle as oracle
+from test_gpu_fsdp2_torch import Block, Toy
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def fake_process_group():
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    def _init(world_size):
+        dist.init_process_group("fake", rank=0, world_size=world_size, store=FakeStore())
+
+    yield _init
+    from odc_amd.fsdp import fsdp1
+
+    fsdp1.unpatch_fsdp1()
+    if dist.is_initialized():
+        dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("W", [4, 8])
+def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, W):
+    from torch.distributed.fsdp import FullyShardedDataParallel as FSDP
+    from torch.distributed.fsdp import MixedPrecision
+    from torch.distributed.fsdp._common_utils import clean_tensor_name
+    from torch.distributed.fsdp.wrap import ModuleWrapPolicy
+
+    from odc_amd import SymmBufferRegistry
+    from odc_amd.fsdp import fsdp1
+
+    fake_process_group(W)
+    group = make_world(W, 64 << 20)
+    fsdp1.patch_fsdp1(reduce_dtype=torch.float32)  # bf16 gradients into fp32 accumulations
+
+    torch.manual_seed(0)
+    model = Toy().cuda()
+    reference = copy.deepcopy(model)
+    full_params = {name: p.detach().clone() for name, p in reference.named_parameters()}
+    fsdp_model = FSDP(
+        model,
+        auto_wrap_policy=ModuleWrapPolicy({Block}),
+        mixed_precision=MixedPrecision(param_dtype=torch.bfloat16),
+        device_id=torch.cuda.current_device(),
+        use_orig_params=False,
+    )
+    units = []  # (handle, [full parameter names in flat order])
+    for name, module in fsdp_model.named_modules():
+        if isinstance(module, FSDP) and module._handle is not None:
+            prefix = clean_tensor_name(name)
+            fqns = [f"{prefix}.{f}" if prefix else f for f in module._handle.flat_param._fqns]
+            units.append((module._handle, fqns))
+    assert len(units) == 4
+    registry = SymmBufferRegistry.get_instance()
+    for handle, fqns in units:
+        flat = torch.cat([full_params[f].reshape(-1) for f in fqns])
+        peers = registry.get_peer_tensors(handle.flat_param.data)
+        for r in range(W):  # every virtual rank's shard was published when the unit was wrapped
+            assert_bit_equal(peers[r], oracle.fsdp1_get_shard(flat, r, W), f"shard {r} of {fqns[0]}...")
+
+    ref_compute = copy.deepcopy(reference).bfloat16()
+    g = torch.Generator().manual_seed(1)
+    batches = [torch.randn(16, 32, generator=g).cuda() for _ in range(3)]
+    pre = fsdp_model._gradient_predivide_factor
+    post = fsdp_model._gradient_postdivide_factor
+    assert pre * post == W
+
+    fsdp1.pre_minibatch_start(fsdp_model)
+    want = [[torch.zeros(h.flat_param.numel()) for _ in range(W)] for h, _ in units]
+    for x in batches:
+        fsdp_model(x).float().pow(2).mean().backward()
+        assert all(h.flat_param.grad is None for h, _ in units)  # published only at the optimizer step
+        ref_compute.zero_grad(set_to_none=True)
+        ref_compute(x.bfloat16()).float().pow(2).mean().backward()
+        grads = {n: p.grad.detach().cpu() for n, p in ref_compute.named_parameters()}
+        for accs, (_, fqns) in zip(want, units):
+            flat_grad = torch.cat([grads[f].reshape(-1) for f in fqns])
+            if pre > 1:
+                flat_grad.div_(pre)  # in bf16, as torch does before the reduce-scatter
+            oracle.scatter_accumulate(accs, oracle.fsdp1_pad_grad(flat_grad, W))
+    fsdp1.pre_optimizer_step(fsdp_model)
+    for accs, (handle, fqns) in zip(want, units):
+        expect = oracle.fsdp1_publish(accs[0].clone(), post, torch.float32)
+        assert handle.flat_param.grad.dtype == torch.float32
+        assert_bit_equal(handle.flat_param.grad, expect, f"flat gradient of {fqns[0]}...")
+
+    opt = torch.optim.SGD(fsdp_model.parameters(), lr=0.1)
+    opt.step()
+    opt.zero_grad()
+    fsdp1.pre_minibatch_start(fsdp_model)
+    out = fsdp_model(batches[0])
+    with torch.no_grad():  # reference: chunk 0 of every flat parameter updated, the rest unchanged
+        named = dict(reference.named_parameters())
+        for handle, fqns in units:
+            flat = torch.cat([named[f].reshape(-1) for f in fqns])
+            S = math.ceil(flat.numel() / W)
+            flat[:S] = handle.flat_param.data[: min(S, flat.numel())]
+            off = 0
+            for f in fqns:
+                named[f].copy_(flat[off : off + named[f].numel()].view_as(named[f]))
+                off += named[f].numel()
+    want_out = copy.deepcopy(reference).bfloat16()(batches[0].bfloat16())
+    assert_bit_equal(out, want_out, "forward after the optimizer step")
