@@ -1,6 +1,5 @@
 """The symmetric arena and registry on the GPU, through the C ABI."""
 
-import ctypes
 
 import pytest
 import torch

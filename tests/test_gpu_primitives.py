@@ -2,7 +2,6 @@
 reference API (which calls the C ABI of libodc_hip.so). Bit-exact: gather is a byte copy;
 scatter-accumulate does one IEEE fp32 add per element per call, in call order."""
 
-import math
 
 import pytest
 import torch
@@ -12,7 +11,7 @@ from oracle import odc_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
-from helpers import assert_bit_equal, bits  # noqa: E402,F401
+from helpers import assert_bit_equal
 
 
 def services():
