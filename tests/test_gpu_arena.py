@@ -112,3 +112,15 @@ def test_gather_from_inner_view_and_multi_item(make_world):
     for r in range(W):
         assert_bit_equal(out_a[r * 100 : (r + 1) * 100], torch.arange(50, 150, dtype=torch.int32) + 10_000 * r)
         assert_bit_equal(out_b[r * 7 : (r + 1) * 7], torch.arange(993, 1000, dtype=torch.int32) + 10_000 * r)
+
+
+def test_plain_c_client_of_the_abi():
+    """tests/c_abi/abi_check.c, built with gcc by build(): the library without Python or torch."""
+    import subprocess
+    from pathlib import Path
+
+    exe = Path(__file__).resolve().parent / "c_abi" / "abi_check"
+    assert exe.exists(), "run `python -c 'import __graft_entry__ as g; g.build()'` first"
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "abi_check ok" in proc.stdout

@@ -28,6 +28,16 @@ def test_library_exports_every_declared_symbol():
     assert _native.MAX_ITEMS_PER_LAUNCH == int(re.search(r"ODC_MAX_ITEMS_PER_LAUNCH (\d+)", header).group(1))
 
 
+def test_header_is_plain_c():
+    import subprocess
+
+    subprocess.run(
+        ["gcc", "-std=c99", "-fsyntax-only", "-Wall", "-Wextra", "-pedantic", "-x", "c",
+         str(ROOT / "include" / "odc_hip.h")],
+        check=True,
+    )
+
+
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_native.GatherItem) == 24
     assert ctypes.sizeof(_native.AccumItem) == 32
