@@ -197,10 +197,14 @@ def load() -> ctypes.CDLL:
     with _lib_lock:
         if _lib is None:
             if not LIB_PATH.exists():
-                raise ImportError(
-                    f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; "
-                    "g.build()'` (needs hipcc). There is no fallback path."
-                )
+                # nothing built yet: build once, in-tree; there is no fallback path
+                try:
+                    build_library()
+                except (OSError, RuntimeError) as e:
+                    raise ImportError(
+                        f"{LIB_PATH} is missing and could not be built ({e}): run "
+                        "`python -c 'import __graft_entry__ as g; g.build()'` (needs hipcc)"
+                    ) from None
             lib = ctypes.CDLL(str(LIB_PATH))
             try:
                 _declare(lib)

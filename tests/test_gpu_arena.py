@@ -120,7 +120,10 @@ def test_plain_c_client_of_the_abi():
     from pathlib import Path
 
     exe = Path(__file__).resolve().parent / "c_abi" / "abi_check"
-    assert exe.exists(), "run `python -c 'import __graft_entry__ as g; g.build()'` first"
+    if not exe.exists():  # nothing built yet
+        import __graft_entry__
+
+        __graft_entry__.build_c_client()
     proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "abi_check ok" in proc.stdout
