@@ -437,8 +437,10 @@ def comm_stream_section():
         yield comm
         return
     comm.wait_stream(current)
-    yield comm
-    current.wait_stream(comm)
+    try:
+        yield comm
+    finally:
+        current.wait_stream(comm)
 
 
 class BufferSplitter:

@@ -1,0 +1,102 @@
+"""Randomised shapes and alignments through the multi-item entry points, against the oracle.
+Every case is seeded; sizes cluster around the tile boundaries (1024 vectors = 16 KiB / 4096
+elements) where head, tail, partial-run and padding logic meet."""
+
+import random
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 2, 3, 5, 15, 16, 17, 63, 64, 65, 255, 1023, 4095, 4096, 4097, 8191, 16383, 16384, 16385,
+         16399, 32768, 32771, 49153, 70001]
+
+
+def pick_size(rng):
+    return rng.choice(SIZES) if rng.random() < 0.8 else rng.randrange(0, 90_000)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_gather_random_byte_layouts(make_world, seed):
+    """uint8 shards at arbitrary byte offsets inside one symmetric buffer, gathered to arbitrary
+    byte offsets inside one output buffer: every alignment combination of both sides."""
+    from odc_amd import GatherService, SymmBufferRegistry
+
+    rng = random.Random(seed)
+    W = rng.choice([1, 2, 3, 5, 8, 12, 16])
+    n_items = rng.choice([1, 2, 7, 33, 40])
+    sizes = [pick_size(rng) for _ in range(n_items)]
+    group = make_world(W, 8 << 20)
+    registry = SymmBufferRegistry.get_instance()
+    src_offs, cursor = [], 0
+    for s in sizes:
+        cursor += rng.randrange(0, 40)
+        src_offs.append(cursor)
+        cursor += s
+    buf_len = cursor + 64
+    registry.allocate_symm_buffer("buf", (buf_len,), torch.uint8)
+    g = torch.Generator().manual_seed(seed)
+    host = [torch.randint(0, 256, (buf_len,), generator=g, dtype=torch.uint8) for _ in range(W)]
+    for r, peer in enumerate(registry.peer_tensors["buf"]):
+        peer.copy_(host[r])
+    local = registry.get_symm_buffer("buf")
+    dst_offs, cursor = [], 0
+    for s in sizes:
+        cursor += rng.randrange(1, 40)
+        dst_offs.append(cursor)
+        cursor += W * s
+    out = torch.full((cursor + 64,), 0xAB, dtype=torch.uint8, device="cuda")
+    outs = [out[o : o + W * s] for o, s in zip(dst_offs, sizes)]
+    ins = [local[o : o + s] for o, s in zip(src_offs, sizes)]
+    GatherService().gather_into_tensors(outs, ins, group)
+    want = torch.full((cursor + 64,), 0xAB, dtype=torch.uint8)
+    for o, so, s in zip(dst_offs, src_offs, sizes):
+        want[o : o + W * s] = oracle.gather([host[r][so : so + s] for r in range(W)])
+    assert_bit_equal(out, want, f"seed {seed}: W={W}, sizes {sizes}")  # also: nothing outside was touched
+
+
+PAIRS = [(torch.bfloat16, torch.float32), (torch.float32, torch.float32), (torch.float16, torch.float32),
+         (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_scatter_accumulate_random_slices_and_padding(make_world, seed):
+    """Several gradients at arbitrary element offsets accumulated into arbitrary slices of one
+    accumulation, each possibly shorter than W * shard (zero padded), twice."""
+    from odc_amd import ReductionService
+
+    rng = random.Random(1000 + seed)
+    W = rng.choice([1, 2, 3, 5, 8, 12, 16])
+    grad_dtype, acc_dtype = PAIRS[seed % len(PAIRS)]
+    n_items = rng.choice([1, 3, 9, 34])
+    sizes = [pick_size(rng) // 4 for _ in range(n_items)]
+    group = make_world(W, 16 << 20)
+    offs, cursor = [], 0
+    for s in sizes:
+        cursor += rng.randrange(0, 9)
+        offs.append(cursor)
+        cursor += s
+    total = cursor + 5
+    valid = [rng.choice([W * s, W * s, max(0, W * s - rng.randrange(0, 50)), rng.randrange(0, W * s + 1)]) for s in sizes]
+    g = torch.Generator().manual_seed(seed)
+    red = ReductionService(accumulation_dtype=acc_dtype)
+    want = [torch.zeros(total, dtype=acc_dtype) for _ in range(W)]
+    for _ in range(2):
+        pool = torch.randn(sum(valid) + 8 * n_items + 8, generator=g).to(grad_dtype)
+        pool_dev = pool.cuda()
+        grads, host_grads, cur = [], [], rng.randrange(0, 8)
+        for v in valid:
+            grads.append(pool_dev[cur : cur + v])
+            host_grads.append(pool[cur : cur + v])
+            cur += v + rng.randrange(0, 8)
+        red.scatter_accumulate_slices("k", grads, offs, sizes, group, accumulation_numel=total)
+        for hg, o, s in zip(host_grads, offs, sizes):
+            padded = torch.cat([hg, torch.zeros(W * s - hg.numel(), dtype=grad_dtype)])
+            oracle.scatter_accumulate([w[o : o + s] for w in want], padded)
+    red.sync(group)
+    for r, acc in enumerate(red.get_peer_accumulations("k")):
+        assert_bit_equal(acc, want[r], f"seed {seed}: W={W} {grad_dtype}->{acc_dtype} rank {r} sizes {sizes} valid {valid}")
