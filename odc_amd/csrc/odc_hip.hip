@@ -564,6 +564,9 @@ template <class A, class O>
 __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch launch) {
   typedef typename Codec<A>::raw_t araw_t;
   typedef typename Codec<O>::raw_t oraw_t;
+  typedef typename Quad<A>::vec_t avec_t;
+  typedef typename Quad<O>::vec_t ovec_t;
+  const uint32_t tid = threadIdx.x;
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
     const TileCoord c = locate_tile(launch.tt, t);
     const uint64_t seg = launch.seg_elems[c.item];
@@ -571,14 +574,36 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
     araw_t* acc = reinterpret_cast<araw_t*>(launch.region + launch.acc_off[c.item]) + in_seg;
     oraw_t* out = launch.out[c.item] ? reinterpret_cast<oraw_t*>(launch.out[c.item]) + in_seg : nullptr;
     const uint64_t left = seg - in_seg;
-    const uint32_t n = left < kTileElems ? (uint32_t)left : kTileElems;
-    for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
-      araw_t raw = acc[i];
-      if (launch.divide) {
-        raw = Codec<A>::narrow(Codec<A>::widen(raw) / launch.divisor);
-        acc[i] = raw;
+    if (left >= kTileElems && (((uintptr_t)acc) & (sizeof(avec_t) - 1)) == 0 &&
+        (((uintptr_t)out) & (sizeof(ovec_t) - 1)) == 0) {
+      avec_t* ap = reinterpret_cast<avec_t*>(acc) + tid;
+      ovec_t* op = reinterpret_cast<ovec_t*>(out) + tid;
+      avec_t raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) raw[u] = __builtin_nontemporal_load(ap + u * kThreads);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        float f[4];
+        Quad<A>::widen(raw[u], f);
+        if (launch.divide) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) f[k] = f[k] / launch.divisor;
+          raw[u] = Quad<A>::narrow(f);
+          __builtin_nontemporal_store(raw[u], ap + u * kThreads);
+          Quad<A>::widen(raw[u], f);  // the copy is a cast of the ROUNDED accumulation
+        }
+        if (out) __builtin_nontemporal_store(Quad<O>::narrow(f), op + u * kThreads);
       }
-      if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw));
+    } else {
+      const uint32_t n = left < kTileElems ? (uint32_t)left : kTileElems;
+      for (uint32_t i = tid; i < n; i += kThreads) {
+        araw_t raw = acc[i];
+        if (launch.divide) {
+          raw = Codec<A>::narrow(Codec<A>::widen(raw) / launch.divisor);
+          acc[i] = raw;
+        }
+        if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw));
+      }
     }
   }
 }
