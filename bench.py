@@ -44,6 +44,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--world-size", type=int, default=8, help="virtual ranks W")
+    ap.add_argument("--workload", choices=["layer", "model"], default="layer",
+                    help="layer: one Llama-3-8B decoder layer (the headline); model: the full 8.03 G "
+                         "parameter model swept unit by unit (needs ~85 GB of HBM; no oracle pass)")
     ap.add_argument("--layout", choices=["per-param", "flat"], default="per-param",
                     help="9 per-parameter shards in one multi-tensor launch, or one flat shard")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -56,12 +59,96 @@ def parse_args():
     return ap.parse_args()
 
 
+def model_sweep(args):
+    """Full Llama-3-8B: per step (= microbatch), gather the 34 FSDP units in forward order, then
+    scatter-accumulate them in reverse order; every 8th step first clears all accumulations."""
+    import torch
+
+    import odc_amd
+    from odc_amd import _native
+    from odc_amd.primitives.utils import get_comm_stream
+    from odc_amd.workloads import llama3_8b_units, numel
+
+    torch.cuda.set_device(0)
+    for opt in args.option:
+        name, value = opt.split("=")
+        _native.set_option(name, int(value))
+    W = args.world_size
+    units = llama3_8b_units()
+    N = sum(numel(s) for _, unit in units for _, s in unit)
+    per_rank = sum((numel(s) // W) * 6 + 512 for _, unit in units for _, s in unit) + (1 << 20)
+    group = odc_amd.init_nvshmem(world_size=W, symmetric_size=per_rank)
+    registry = odc_amd.SymmBufferRegistry.get_instance()
+    gather = odc_amd.GatherService()
+    reduction = odc_amd.ReductionService(accumulation_dtype=torch.float32)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    by_shape = {}  # unit signature -> (output buffers, two sets of gradients): reused across layers
+    plan = []
+    for u, (_, unit) in enumerate(units):
+        sig = tuple(numel(s) for _, s in unit)
+        if sig not in by_shape:
+            outs = [torch.empty(n, dtype=torch.bfloat16, device="cuda") for n in sig]
+            grads = [[(torch.randn(n, generator=gen, device="cuda") * 1e-3).bfloat16() for n in sig] for _ in range(2)]
+            by_shape[sig] = (outs, grads)
+        keys = [(u, p) for p in range(len(unit))]
+        for key, n in zip(keys, sig):
+            registry.allocate_symm_buffer(key, (n // W,), torch.bfloat16)
+            for peer in registry.peer_tensors[key]:
+                peer.normal_(0.0, 0.02, generator=gen)
+            reduction.register(key, (n // W,), torch.bfloat16, torch.float32, group)
+        plan.append((keys, [registry.get_symm_buffer(k) for k in keys], *by_shape[sig]))
+    torch.cuda.synchronize()
+    comm = get_comm_stream()
+
+    def step(i):
+        if i % MICROBATCHES == 0:
+            reduction.clear_accumulations()
+        for keys, locals_, outs, grads in plan:
+            gather.gather_into_tensors(outs, locals_, group)
+        for keys, locals_, outs, grads in reversed(plan):
+            reduction.scatter_accumulate_multi(keys, grads[i % 2], group)
+
+    gc.collect()
+    gc.disable()
+    with torch.cuda.stream(comm):
+        for i in range(args.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(comm)
+        for i in range(args.steps):
+            step(i)
+        e1.record(comm)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    gc.enable()
+    value = args.steps * 14 * N / elapsed / 1e9
+    print(json.dumps({
+        "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for gather + scatter-accum, full 8B model sweep, W=8",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"cfg5: full Llama-3-8B ({N} bf16 params, {len(units)} units, {2 * len(units)} "
+                               f"launches per step), W={W} virtual shards", "world_size": W, "elements": N,
+                   "bytes_per_step": 14 * N},
+        "frac_of_peak": round(value / HBM_PEAK_GBPS, 4),
+        "gpu_ms_per_step": round(e0.elapsed_time(e1) / args.steps, 3),
+        "roofline": None, "cpu_baseline": None, "parity_vs_oracle": None,
+    }))
+    torch.cuda.synchronize()
+    registry.finalize()
+    odc_amd.finalize_distributed()
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: W virtual ranks share one MI355X and nothing here uses a "
               "second GPU. Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "model":
+        return model_sweep(args)
 
     import torch
 
