@@ -266,3 +266,39 @@ def test_publish_divides_in_place_and_casts(make_world, divisor, out_dtype):
                 assert out.data_ptr() == reduction.get_accumulation(k).data_ptr()  # no copy, like .to()
     for r in (0, 1, 3):  # other ranks untouched
         assert_bit_equal(reduction.get_peer_accumulations("a")[r], want["a"][r], f"rank {r}")
+
+
+def test_every_virtual_rank_as_a_client(make_world):
+    """examples/reduce_scatter.py:96-105,163-172 on one GPU: each of the W ranks scatter-accumulates
+    its own gradient, one after the other, for several rounds; rank r's accumulation then equals
+    the reduce-scatter sum of chunk r over clients, accumulated over rounds (within the reference's
+    rtol=atol=5e-3, and bit for bit equal to the oracle run in the same client order). Gathers
+    issued from every rank's point of view give the same result."""
+    from odc_amd import virtual_rank
+
+    W, S, rounds = 8, 16 * 1024 + 128, 4
+    group = make_world(W, 16 << 20)
+    gather, reduction, registry = services()
+    g = torch.Generator().manual_seed(21)
+    want = [torch.zeros(S) for _ in range(W)]
+    nccl_like = [torch.zeros(S) for _ in range(W)]
+    for _ in range(rounds):
+        client_grads = [torch.rand(W * S, generator=g) for _ in range(W)]  # fp32 grads, as the example
+        for q in range(W):
+            with virtual_rank(q):
+                reduction.scatter_accumulate(0, client_grads[q].cuda(), group)
+            oracle.scatter_accumulate(want, client_grads[q])
+        reduced = torch.stack(client_grads).sum(0).view(W, S)  # reduce_scatter(SUM) ...
+        for r in range(W):
+            nccl_like[r].add_(reduced[r])  # ... followed by add_
+    reduction.sync(group)
+    for r, acc in enumerate(reduction.get_peer_accumulations(0)):
+        assert_bit_equal(acc, want[r], f"rank {r}")
+        torch.testing.assert_close(acc.cpu(), nccl_like[r], rtol=5e-3, atol=5e-3)
+    shards = [torch.randn(S, generator=g).bfloat16() for _ in range(W)]
+    put_shards(registry, "p", shards, group)
+    for q in range(W):
+        with virtual_rank(q):
+            out = torch.empty(W * S, dtype=torch.bfloat16, device="cuda")
+            gather.gather_into_tensor(out, registry.get_symm_buffer("p"), group)
+            assert_bit_equal(out, oracle.gather(shards), f"gather as rank {q}")
