@@ -62,6 +62,14 @@ def test_fsdp1_hooks_and_call_sites(make_world):
     for h in handles:
         acc = fsdp1.get_reduction_service().get_accumulation(id(h.flat_param))
         assert not acc.cpu().any()
+    # stop() tears everything down (fsdp1.py:345-348)
+    from odc_amd.primitives import utils
+
+    for h in handles:
+        h.flat_param.data = torch.empty(0)  # drop the views into the arena first
+        h.flat_param.grad = None
+    fsdp1.stop()
+    assert not utils.is_initialized() and not odc_amd.SymmBufferRegistry.get_instance().has_key(id(handles[0].flat_param))
 
 
 @pytest.mark.parametrize("W", [4, 8, 12])
@@ -113,3 +121,8 @@ def test_fsdp2_group_layout(make_world, W, fused, dtype):
                 assert tuple(a.shape) == tuple(b.shape), f"rank {r} param {p}"
                 assert_bit_equal(a.contiguous(), b.contiguous(), f"rank {r} sharded grad {p}")
     assert set(fsdp2.get_symm_buffer_memory_breakdown()) >= {"fsdp_params", "accumulation"}
+    from odc_amd.primitives import utils
+
+    del got, unsharded, pgp
+    fsdp2.stop()  # fsdp2.py:1141-1144
+    assert not utils.is_initialized()
