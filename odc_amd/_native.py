@@ -16,7 +16,8 @@ from pathlib import Path
 _PKG_DIR = Path(__file__).resolve().parent
 CSRC_DIR = _PKG_DIR / "csrc"
 INCLUDE_DIR = _PKG_DIR.parent / "include"
-LIB_PATH = CSRC_DIR / "libodc_hip.so"
+# $ODC_HIP_LIBRARY points at a library built elsewhere (same ABI); default: the in-tree build
+LIB_PATH = Path(os.environ["ODC_HIP_LIBRARY"]) if os.environ.get("ODC_HIP_LIBRARY") else CSRC_DIR / "libodc_hip.so"
 SOURCES = [CSRC_DIR / "odc_hip.hip"]
 
 # every symbol include/odc_hip.h declares
