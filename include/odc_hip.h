@@ -191,11 +191,14 @@ int odc_publish(odc_arena* arena, uint32_t rank, const odc_publish_item* items, 
 const char* odc_last_error(void);
 int odc_abi_version(void);
 
-/* Launch-shape knobs, for measurement. Names: "gather_blocks_per_cu", "accum_blocks_per_cu",
- * "clear_blocks_per_cu" (0 = one block per tile, no grid-stride loop), "rank_major" (gather and
- * scatter-accumulate: 1 = walk a rank's whole shard before the next rank, 0 = interleave ranks
- * tile by tile), "rank_stagger_bytes" (extra distance between rank regions, read when an arena
- * is created). Unknown names return ODC_ERR_INVALID. Results never depend on these. */
+/* Launch-shape knobs, for measurement. "gather_blocks_per_cu", "accum_blocks_per_cu",
+ * "clear_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
+ * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
+ * "accum_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per CU
+ * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather and scatter-accumulate:
+ * 1 = walk a rank's whole shard before the next rank, 0 = interleave ranks tile by tile);
+ * "rank_stagger_bytes" (extra distance between rank regions, read when an arena is created).
+ * Unknown names return ODC_ERR_INVALID. Results never depend on these. */
 int odc_set_option(const char* name, int64_t value);
 int odc_get_option(const char* name, int64_t* value);
 

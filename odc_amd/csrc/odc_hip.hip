@@ -62,9 +62,12 @@ int fail(int code, const char* fmt, ...) {
 // options
 // ------------------------------------------------------------------------------------------------
 struct Options {
-  // measured on MI355X over a Llama-3-8B layer: gather peaks at 2 workgroups per CU, the
-  // read-modify-write at 1, the pure-write clear with one workgroup per tile
-  int64_t gather_blocks_per_cu = 2;
+  // measured on MI355X over a Llama-3-8B layer: the gather peaks with one workgroup per tile and
+  // at most 4 of them resident per CU, the read-modify-write with 1 persistent workgroup per CU,
+  // the pure-write clear with one workgroup per tile
+  int64_t gather_blocks_per_cu = 0;
+  int64_t gather_resident_cap = 4;
+  int64_t accum_resident_cap = 4;  // only ragged launches run one workgroup per tile
   int64_t accum_blocks_per_cu = 1;
   int64_t clear_blocks_per_cu = 0;
   int64_t rank_major = 1;
@@ -80,6 +83,8 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
   if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
+  if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
+  if (!strcmp(name, "accum_resident_cap")) return &g_opt.accum_resident_cap;
   return nullptr;
 }
 
@@ -622,6 +627,8 @@ struct odc_arena {
   int device = -1;
   uint32_t flags = 0;
   int n_cu = 256;
+  int lds_per_cu = 160 * 1024;
+  int lds_per_wg_max = 64 * 1024;
   uint64_t bytes_per_rank = 0;
   uint64_t rank_stride = 0;
   uint8_t* base = nullptr;
@@ -684,6 +691,16 @@ uint32_t grid_for(const odc_arena* a, int64_t blocks_per_cu, uint32_t n_tiles, b
   return (uint32_t)std::min<uint64_t>(g, n_tiles);
 }
 
+// One-workgroup-per-tile launches are dealt out by the hardware dispatcher, which keeps as many
+// workgroups resident as fit. Fewer resident workgroups (a smaller window of memory in flight)
+// can stream faster; the only lever is to make each workgroup claim a share of the CU's LDS that
+// it never touches. Returns the dynamic LDS bytes that leave room for exactly `cap` workgroups.
+uint32_t lds_claim_for(const odc_arena* a, int64_t cap, uint32_t grid, uint32_t n_tiles) {
+  if (cap <= 0 || grid != n_tiles) return 0;  // persistent grids size themselves
+  const uint64_t per_wg = ((uint64_t)a->lds_per_cu / (uint64_t)cap) & ~(uint64_t)1023;
+  return (uint32_t)std::min<uint64_t>(per_wg, (uint64_t)a->lds_per_wg_max);
+}
+
 constexpr uint64_t kMaxTilesPerLaunch = 1ull << 31;
 
 }  // namespace
@@ -731,6 +748,14 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
   if (!(flags & ODC_ARENA_NO_BACKING)) {
     hipError_t e = hipGetDevice(&a->device);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&a->n_cu, hipDeviceAttributeMultiprocessorCount, a->device);
+    if (e == hipSuccess) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, a->device) == hipSuccess && v > 0)
+        a->lds_per_cu = v;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, a->device) == hipSuccess && v > 0)
+        a->lds_per_wg_max = v;
+      (void)hipGetLastError();
+    }
     void* p = nullptr;
     if (e == hipSuccess) e = hipMalloc(&p, a->rank_stride * world_size);
     if (e != hipSuccess) {
@@ -1016,7 +1041,8 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
       ragged |= (((uintptr_t)L.dst[k] | L.src_off[k] | L.seg_bytes[k]) & 15u) != 0;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles, ragged);
-    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles),
+                       static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;
@@ -1063,7 +1089,8 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     if (n < 0) return n;
     if (n == 0) continue;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles),
+                       static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;
@@ -1152,7 +1179,8 @@ int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n
       ragged |= (L.acc_off[k] & 15u) != 0 || (L.seg_elems[k] & 3u) != 0 ||
                 ((uintptr_t)L.grad[k] & (4u * gb - 1)) != 0 || L.grad_elems[k] != L.seg_elems[k] * a->world;
     const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.accum_resident_cap, grid, L.tt.n_tiles),
+                       static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;
