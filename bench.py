@@ -33,8 +33,8 @@ MICROBATCHES = 8
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE and
 # WRITE_SIZE runs, scaled by a torch copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("accum", "per-param", 8): 2_181_124_225,
-    ("gather", "per-param", 8): 872_479_914,
+    ("accum", "per-param", 8): 2_181_147_164,
+    ("gather", "per-param", 8): 872_533_161,
 }
 
 
