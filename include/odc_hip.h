@@ -194,7 +194,7 @@ int odc_abi_version(void);
 /* Launch-shape knobs, for measurement. "gather_blocks_per_cu", "accum_blocks_per_cu",
  * "clear_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
  * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
- * "accum_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per CU
+ * "cast_resident_cap", "accum_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per CU
  * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather and scatter-accumulate:
  * 1 = walk a rank's whole shard before the next rank, 0 = interleave ranks tile by tile);
  * "rank_stagger_bytes" (extra distance between rank regions, read when an arena is created).

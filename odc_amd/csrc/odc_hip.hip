@@ -67,6 +67,7 @@ struct Options {
   // the pure-write clear with one workgroup per tile
   int64_t gather_blocks_per_cu = 0;
   int64_t gather_resident_cap = 4;
+  int64_t cast_resident_cap = 0;  // the read-heavy converting gather streams best uncapped
   int64_t accum_resident_cap = 4;  // only ragged launches run one workgroup per tile
   int64_t accum_blocks_per_cu = 1;
   int64_t clear_blocks_per_cu = 0;
@@ -84,6 +85,7 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
   if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
   if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
+  if (!strcmp(name, "cast_resident_cap")) return &g_opt.cast_resident_cap;
   if (!strcmp(name, "accum_resident_cap")) return &g_opt.accum_resident_cap;
   return nullptr;
 }
@@ -1089,7 +1091,7 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     if (n < 0) return n;
     if (n == 0) continue;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles),
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.cast_resident_cap, grid, L.tt.n_tiles),
                        static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
