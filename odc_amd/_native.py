@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "odc_gather",
     "odc_gather_cast",
     "odc_scatter_accumulate",
+    "odc_scatter_store",
     "odc_clear",
     "odc_publish",
     "odc_last_error",
@@ -179,6 +180,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.odc_gather.argtypes = [vp, P(GatherItem), u32, u32, vp]
     lib.odc_gather_cast.argtypes = [vp, P(GatherCastItem), u32, ci, ci, u32, vp]
     lib.odc_scatter_accumulate.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
+    lib.odc_scatter_store.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
     lib.odc_publish.argtypes = [vp, u32, P(PublishItem), u32, ci, ci, ctypes.c_float, vp]
     lib.odc_clear.argtypes = [vp, P(Span), u32, vp]
     lib.odc_last_error.argtypes = []

@@ -4,6 +4,7 @@
 //   gather_kernel       : W shard regions -> one flat buffer          (read 1 B + write 1 B per byte)
 //   cast_gather_kernel  : the same with a dtype conversion on the way (fp32 -> bf16: 6 B per element)
 //   accum_kernel        : acc_r += widen(grad chunk r), in place      (bf16 -> fp32: 10 B per element)
+//                         or acc_r = +0 + widen(grad chunk r), acc not read          (6 B per element)
 //   clear_kernel        : zero a span in every rank region            (write 1 B per byte)
 //   publish_kernel      : one rank's acc /= divisor, plus a cast copy (end of a minibatch)
 // plus the host-side symmetric arena (one hipMalloc, W rank regions, one offset valid in all).
@@ -70,6 +71,8 @@ struct Options {
   int64_t cast_resident_cap = 0;  // the read-heavy converting gather streams best uncapped
   int64_t accum_resident_cap = 4;  // only ragged launches run one workgroup per tile
   int64_t accum_blocks_per_cu = 1;
+  int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
+  int64_t store_resident_cap = 4;
   int64_t clear_blocks_per_cu = 0;
   int64_t rank_major = 1;
   int64_t rank_stagger_bytes = 0;
@@ -87,6 +90,8 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
   if (!strcmp(name, "cast_resident_cap")) return &g_opt.cast_resident_cap;
   if (!strcmp(name, "accum_resident_cap")) return &g_opt.accum_resident_cap;
+  if (!strcmp(name, "store_blocks_per_cu")) return &g_opt.store_blocks_per_cu;
+  if (!strcmp(name, "store_resident_cap")) return &g_opt.store_resident_cap;
   return nullptr;
 }
 
@@ -396,7 +401,9 @@ template <> struct Quad<f16_tag> {
   }
 };
 
-template <class G, class A>
+// kStore: the accumulation is taken to hold +0 and is not read (acc = +0 + g, the value a clear
+// followed by an accumulate leaves: -0 gradients still become +0).
+template <class G, class A, bool kStore>
 __device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uint64_t gi,
                                           uint64_t grad_elems, uint64_t i) {
   typedef typename Codec<A>::raw_t araw_t;
@@ -404,18 +411,20 @@ __device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uin
   araw_t* a = reinterpret_cast<araw_t*>(acc) + i;
   float g = 0.0f;  // padding reads as +0 and is still added (so -0 + +0 -> +0, as F.pad + add_)
   if (gi < grad_elems) g = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi]);
-  *a = Codec<A>::narrow(Codec<A>::widen(*a) + g);
+  float before = 0.0f;
+  if constexpr (!kStore) before = Codec<A>::widen(*a);
+  *a = Codec<A>::narrow(before + g);
 }
 
 // One quad (4 elements) of a tile that is partial, crosses the end of the valid gradient, or
 // lies in the zero padding. acc points at the quad, gi is its first element's gradient index.
-template <class G, class A>
+template <class G, class A, bool kStore>
 __device__ __forceinline__ void accum_quad_guarded(uint8_t* acc, const uint8_t* grad, uint64_t gi,
                                                    uint64_t grad_elems) {
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
   avec_t* ap = reinterpret_cast<avec_t*>(acc);
-  float gf[4] = {0.0f, 0.0f, 0.0f, 0.0f}, af[4];
+  float gf[4] = {0.0f, 0.0f, 0.0f, 0.0f}, af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if (gi + 4 <= grad_elems) {
     Quad<G>::widen(load_stream<gvec_t>(grad + gi * Codec<G>::kBytes), gf);
   } else {
@@ -424,7 +433,7 @@ __device__ __forceinline__ void accum_quad_guarded(uint8_t* acc, const uint8_t* 
     for (int k = 0; k < 4; ++k)
       if (gi + k < grad_elems) gf[k] = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi + k]);
   }
-  Quad<A>::widen(__builtin_nontemporal_load(ap), af);
+  if constexpr (!kStore) Quad<A>::widen(__builtin_nontemporal_load(ap), af);
 #pragma unroll
   for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
   __builtin_nontemporal_store(Quad<A>::narrow(af), ap);
@@ -432,7 +441,7 @@ __device__ __forceinline__ void accum_quad_guarded(uint8_t* acc, const uint8_t* 
 
 // The parts of a tile that are not whole runs of valid quads: a partial last run, a run that
 // crosses the end of the valid gradient or lies in the zero padding, the head and the tail.
-template <class G, class A>
+template <class G, class A, bool kStore>
 __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_t* grad, uint64_t g_seg,
                                                       uint64_t grad_elems, uint32_t chunk, SegShape g,
                                                       bool body) {
@@ -446,17 +455,17 @@ __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_
     for (int u = 0; u < kUnroll; ++u) {
       const uint32_t q = u * kThreads + tid;
       if (q < left)
-        accum_quad_guarded<G, A>(acc + (e0 + (uint64_t)q * 4) * kAB, grad, g_seg + e0 + (uint64_t)q * 4, grad_elems);
+        accum_quad_guarded<G, A, kStore>(acc + (e0 + (uint64_t)q * 4) * kAB, grad, g_seg + e0 + (uint64_t)q * 4, grad_elems);
     }
   }
-  if (chunk == 0 && tid < g.head) accum_one<G, A>(acc, grad, g_seg + tid, grad_elems, tid);
+  if (chunk == 0 && tid < g.head) accum_one<G, A, kStore>(acc, grad, g_seg + tid, grad_elems, tid);
   if (chunk == g.last && tid < g.tail) {
     const uint64_t i = g.head + g.nvec * 4 + tid;
-    accum_one<G, A>(acc, grad, g_seg + i, grad_elems, i);
+    accum_one<G, A, kStore>(acc, grad, g_seg + i, grad_elems, i);
   }
 }
 
-template <class G, class A>
+template <class G, class A, bool kStore>
 __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launch) {
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
@@ -480,20 +489,22 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
       avec_t araw[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) graw[u] = load_stream<gvec_t>(gb + (size_t)u * kThreads * sizeof(gvec_t));
+      if constexpr (!kStore) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) araw[u] = __builtin_nontemporal_load(ap + u * kThreads);
+        for (int u = 0; u < kUnroll; ++u) araw[u] = __builtin_nontemporal_load(ap + u * kThreads);
+      }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        float gf[4], af[4];
+        float gf[4], af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         Quad<G>::widen(graw[u], gf);
-        Quad<A>::widen(araw[u], af);
+        if constexpr (!kStore) Quad<A>::widen(araw[u], af);
 #pragma unroll
         for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
         __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * kThreads);
       }
     }
     if (!whole || (c.chunk == 0 && g.head) || (c.chunk == g.last && g.tail))
-      accum_edges<G, A>(acc, grad, g_seg, grad_elems, c.chunk, g, !whole);
+      accum_edges<G, A, kStore>(acc, grad, g_seg, grad_elems, c.chunk, g, !whole);
   }
 }
 
@@ -983,8 +994,9 @@ typedef void (*publish_fn)(const PublishLaunch);
   X(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F16, f16_tag)     \
   X(ODC_DTYPE_F32, f32_tag, ODC_DTYPE_F32, f32_tag)
 
-accum_fn pick_accum(int g, int a) {  // (gradient dtype, accumulation dtype)
-#define X(E1, T1, E2, T2) if (g == E1 && a == E2) return accum_kernel<T1, T2>;
+accum_fn pick_accum(int g, int a, bool store) {  // (gradient dtype, accumulation dtype)
+#define X(E1, T1, E2, T2) \
+  if (g == E1 && a == E2) return store ? accum_kernel<T1, T2, true> : accum_kernel<T1, T2, false>;
   ODC_FOR_EACH_DTYPE_PAIR(X)
 #undef X
   return nullptr;
@@ -1127,14 +1139,19 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
   return ODC_OK;
 }
 
-int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
-                           int grad_dtype, int acc_dtype, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// odc_scatter_accumulate (store == false) and odc_scatter_store (store == true)
+int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, int grad_dtype,
+                   int acc_dtype, void* stream, bool store) {
   DeviceGuard guard;
   if (int rc = check_compute(a, guard)) return rc;
   if (n_items && !items) return fail(ODC_ERR_INVALID, "items is NULL");
   const int gb = dtype_bytes(grad_dtype), ab = dtype_bytes(acc_dtype);
   if (!gb || !ab) return fail(ODC_ERR_INVALID, "unknown dtype code (grad %d, acc %d)", grad_dtype, acc_dtype);
-  const accum_fn kernel = pick_accum(grad_dtype, acc_dtype);
+  const accum_fn kernel = pick_accum(grad_dtype, acc_dtype, store);
   if (!kernel)
     return fail(ODC_ERR_UNSUPPORTED, "scatter-accumulate of grad dtype %d into acc dtype %d is not implemented",
                 grad_dtype, acc_dtype);
@@ -1180,12 +1197,28 @@ int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
       ragged |= (L.acc_off[k] & 15u) != 0 || (L.seg_elems[k] & 3u) != 0 ||
                 ((uintptr_t)L.grad[k] & (4u * gb - 1)) != 0 || L.grad_elems[k] != L.seg_elems[k] * a->world;
-    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.accum_resident_cap, grid, L.tt.n_tiles),
+    const uint32_t grid =
+        grid_for(a, store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
+    const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, cap, grid, L.tt.n_tiles),
                        static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int odc_scatter_accumulate(odc_arena* a, const odc_accum_item* items, uint32_t n_items,
+                           int grad_dtype, int acc_dtype, void* stream) {
+  return scatter_launch(a, items, n_items, grad_dtype, acc_dtype, stream, false);
+}
+
+int odc_scatter_store(odc_arena* a, const odc_accum_item* items, uint32_t n_items, int grad_dtype,
+                      int acc_dtype, void* stream) {
+  return scatter_launch(a, items, n_items, grad_dtype, acc_dtype, stream, true);
 }
 
 int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint32_t n_items,

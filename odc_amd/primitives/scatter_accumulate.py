@@ -7,12 +7,21 @@ reference the caller copies chunk r into a staging buffer on rank r (:649-669), 
 (:369-395). With every rank's accumulation in one HBM the owner is the caller, so staging,
 doorbells and the watcher collapse into ``odc_scatter_accumulate`` (include/odc_hip.h): one read
 of the gradient, one read-modify-write of the accumulations.
+
+Clears are lazy by default: ``clear_accumulations`` only notes that every accumulation now counts
+as zero, and the first scatter-accumulate of a key after it runs as ``odc_scatter_store``
+(``acc = +0 + grad``, the accumulation is written but never read). The bits are those of a clear
+followed by an accumulate; per minibatch it saves the clear's 4 bytes per element and the first
+read of the accumulation (4 more). Whatever hands an accumulation out (``get_accumulation``,
+``get_peer_accumulations``, ``publish``) first writes the zeros that are still owed.
+``ReductionService(lazy_clear=False)`` or ``ODC_LAZY_CLEAR=0`` clears eagerly.
 """
 
 from __future__ import annotations
 
 import ctypes
 import logging
+import os
 from typing import Sequence
 
 import torch
@@ -33,12 +42,16 @@ logger = logging.getLogger(__name__)
 
 
 class ReductionService:
-    def __init__(self, accumulation_dtype=None):
+    def __init__(self, accumulation_dtype=None, lazy_clear=None):
         self.accumulations = []  # index -> key (tensors come from the registry, per rank)
         self.accumulation_indices = {}
         self.accumulation_dtype = accumulation_dtype
         self.dispatched_tasks = 0
         self.buffer_splitter = BufferSplitter()
+        if lazy_clear is None:
+            lazy_clear = os.environ.get("ODC_LAZY_CLEAR", "1") != "0"
+        self.lazy_clear = bool(lazy_clear)
+        self._owed_zero = set()  # keys whose accumulations count as zero but hold stale bytes
 
     # -- registration ---------------------------------------------------------------------
     @staticmethod
@@ -58,9 +71,14 @@ class ReductionService:
         registry.allocate_symm_buffer(accumulation_key, tuple(output_tensor_shape), reduction_dtype)
         self.accumulation_indices[key] = len(self.accumulations)
         self.accumulations.append(key)
-        self._clear_keys([key])
+        if self.lazy_clear:
+            self._owed_zero.add(key)
+        else:
+            self._clear_keys([key])
 
     def _clear_keys(self, keys):
+        keys = list(keys)
+        self._owed_zero.difference_update(keys)
         if not keys:
             return
         registry = SymmBufferRegistry.get_instance()
@@ -80,8 +98,35 @@ class ReductionService:
         """Zero every registered accumulation of EVERY virtual rank in one launch
         (``acc.fill_(0)`` per key and per process in the reference, :585-587). Idempotent, so
         each virtual rank may call it; like there, no rank may have started the minibatch's
-        scatter-accumulates before the last clear."""
-        self._clear_keys(self.accumulations)
+        scatter-accumulates before the last clear. Lazy mode launches nothing here."""
+        # under stream capture the clear must be a kernel in the graph, not host-side state
+        if self.lazy_clear and not torch.cuda.is_current_stream_capturing():
+            self._owed_zero.update(self.accumulations)
+        else:
+            self._clear_keys(self.accumulations)
+
+    def _settle(self, keys):
+        """Write the zeros still owed to ``keys`` (before anything reads or adds into them)."""
+        owed = [k for k in keys if k in self._owed_zero]
+        if owed:
+            self._clear_keys(owed)
+
+    def _launch(self, items, grad_dtype, acc_dtype, store):
+        if not len(items):
+            return
+        lib = _native.load()
+        entry = lib.odc_scatter_store if store else lib.odc_scatter_accumulate
+        with comm_stream_section() as comm:
+            _native.check(
+                entry(
+                    get_world().arena.handle,
+                    items,
+                    len(items),
+                    native_dtype(grad_dtype),
+                    native_dtype(acc_dtype),
+                    ctypes.c_void_p(comm.cuda_stream),
+                )
+            )
 
     # -- the primitive ----------------------------------------------------------------------
     def infer_output_shape(self, input_tensor, pg):
@@ -139,17 +184,25 @@ class ReductionService:
             items[i].acc_offset = offset
             items[i].shard_elems = shard_shape[0]
 
-        with comm_stream_section() as comm:
-            _native.check(
-                _native.load().odc_scatter_accumulate(
-                    world.arena.handle,
-                    items,
-                    len(items),
-                    native_dtype(grad_dtype),
-                    native_dtype(acc_dtype),
-                    ctypes.c_void_p(comm.cuda_stream),
-                )
-            )
+        # Keys that still count as zero take the store form (no read of the accumulation). A key
+        # listed k times goes into k consecutive launches, so its gradients add up in list order.
+        rounds, times_seen = [], {}
+        for i, key in enumerate(keys):
+            k = times_seen.get(key, 0)
+            times_seen[key] = k + 1
+            if k == len(rounds):
+                rounds.append([])
+            rounds[k].append(i)
+        for k, members in enumerate(rounds):
+            for store in (True, False):
+                picked = [i for i in members if (k == 0 and keys[i] in self._owed_zero) == store]
+                if not picked:
+                    continue
+                part = items
+                if len(picked) != len(items):
+                    part = (_native.AccumItem * len(picked))(*[items[i] for i in picked])
+                self._launch(part, grad_dtype, acc_dtype, store)
+        self._owed_zero.difference_update(keys)
         self.dispatched_tasks += len(items)
 
     def scatter_accumulate_slices(
@@ -193,17 +246,22 @@ class ReductionService:
             items[i].grad_elems = grad.numel()
             items[i].acc_offset = offset + off * acc_dtype.itemsize
             items[i].shard_elems = n
-        with comm_stream_section() as comm:
-            _native.check(
-                _native.load().odc_scatter_accumulate(
-                    world.arena.handle,
-                    items,
-                    len(items),
-                    native_dtype(grad_dtype),
-                    native_dtype(acc_dtype),
-                    ctypes.c_void_p(comm.cuda_stream),
-                )
-            )
+        store = False
+        if key in self._owed_zero:
+            # the store form needs the slices to tile the whole accumulation exactly once
+            spans = sorted((int(o), int(n)) for o, n in zip(slice_offsets, slice_numels) if n)
+            end = 0
+            for o, n in spans:
+                if o != end:
+                    break
+                end = o + n
+            else:
+                store = end == acc_shape[0]
+            if store:
+                self._owed_zero.discard(key)
+            else:
+                self._settle([key])
+        self._launch(items, grad_dtype, acc_dtype, store)
         self.dispatched_tasks += 1
 
     # -- results ----------------------------------------------------------------------------
@@ -212,6 +270,7 @@ class ReductionService:
         ``odc/fsdp/fsdp2.py:846-847``)."""
         if key not in self.accumulation_indices:
             raise KeyError(key)
+        self._settle([key])
         return SymmBufferRegistry.get_instance().get_symm_buffer(self._acc_key(key))
 
     def publish(self, keys: Sequence, out_dtype=None, divisor: float = 1.0):
@@ -222,6 +281,7 @@ class ReductionService:
         ``odc/fsdp/fsdp1.py:324-335``; ``odc/fsdp/fsdp2.py:846-847,897-899``."""
         if not keys:
             return []
+        self._settle(keys)
         registry = SymmBufferRegistry.get_instance()
         items = (_native.PublishItem * len(keys))()
         results, acc_dtype = [], None
@@ -255,8 +315,13 @@ class ReductionService:
             )
         return results
 
+    def _registry_peers(self, key):
+        """The W accumulation buffers as they are in memory (owed zeros not written)."""
+        return SymmBufferRegistry.get_instance().peer_tensors[self._acc_key(key)]
+
     def get_peer_accumulations(self, key):
         """All W ranks' accumulation buffers for ``key`` (virtual-world convenience)."""
+        self._settle([key])
         return SymmBufferRegistry.get_instance().peer_tensors[self._acc_key(key)]
 
     def sync(self, pg=None):

@@ -86,6 +86,17 @@ int main(void) {
       CHECK(memcmp(&host_acc[i], (const void*)&want, 4) == 0);
     }
   }
+  /* scatter-store over the stale sums: as if cleared first, then accumulated once */
+  CHECK(odc_scatter_store(arena, &ai, 1, ODC_DTYPE_BF16, ODC_DTYPE_F32, NULL) == ODC_OK);
+  CHECK(hipDeviceSynchronize() == hipSuccess);
+  for (int r = 0; r < W; ++r) {
+    CHECK(hipMemcpy(host_acc, odc_arena_ptr(arena, (uint32_t)r, acc_off), S * 4, hipMemcpyDeviceToHost) == hipSuccess);
+    for (int i = 0; i < S; ++i) {
+      const uint64_t g = (uint64_t)r * S + i;
+      volatile float want = 0.0f + (g < valid ? widen(host_full[g]) : 0.0f);
+      CHECK(memcmp(&host_acc[i], (const void*)&want, 4) == 0);
+    }
+  }
   CHECK(odc_clear(arena, &span, 1, NULL) == ODC_OK);
   CHECK(hipDeviceSynchronize() == hipSuccess);
   for (int r = 0; r < W; ++r) {

@@ -1,0 +1,194 @@
+"""The store form of scatter-accumulate (first accumulate after a clear, without the clear) and
+the lazy clear built on it: the bits must be those of ``acc.fill_(0)`` followed by ``acc.add_``
+(odc/primitives/scatter_accumulate.py:585-587, :386), and the accumulation must not be read."""
+
+import ctypes
+import random
+
+import pytest
+import torch
+
+from helpers import assert_bit_equal
+from oracle import odc_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+PAIRS = [(torch.bfloat16, torch.float32), (torch.float32, torch.float32), (torch.float16, torch.float32),
+         (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.bfloat16),
+         (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16), (torch.float32, torch.float16)]
+
+
+def poison(acc_peers):
+    """Fill accumulations with NaN bit patterns: any read of them would show in the result."""
+    for peer in acc_peers:
+        peer.view(torch.uint8).fill_(0xFF)
+
+
+@pytest.mark.parametrize("grad_dtype,acc_dtype", PAIRS)
+@pytest.mark.parametrize("W,S,valid_short", [(1, 5, 0), (4, 1, 1), (8, 4096, 0), (8, 4099, 13), (12, 33_337, 40_000),
+                                             (3, 70_001, 3)])
+def test_scatter_store_through_the_c_abi(make_world, grad_dtype, acc_dtype, W, S, valid_short):
+    """odc_scatter_store over poisoned accumulations equals zeros + one oracle accumulate; the
+    bytes around the accumulation slices stay as they were."""
+    from odc_amd import SymmBufferRegistry, _native
+    from odc_amd.primitives.utils import get_world, native_dtype
+
+    make_world(W, 4 << 20)
+    registry = SymmBufferRegistry.get_instance()
+    guard = 7  # elements kept on both sides of the slice the store writes
+    registry.allocate_symm_buffer("acc", (S + 2 * guard,), acc_dtype)
+    peers = registry.peer_tensors["acc"]
+    poison(peers)
+    offset = registry.get_offset("acc") + guard * acc_dtype.itemsize
+    g = torch.Generator().manual_seed(S + W)
+    valid = max(0, W * S - valid_short)
+    grad = torch.randn(valid + 3, generator=g).to(grad_dtype)
+    grad[::5] = -0.0
+    dev = grad.cuda()[3:]  # an odd element offset on the gradient side too
+    assert dev.numel() == valid
+    item = _native.AccumItem(dev.data_ptr(), valid, offset, S)
+    items = (_native.AccumItem * 1)(item)
+    _native.check(_native.load().odc_scatter_store(
+        get_world().arena.handle, items, 1, native_dtype(grad_dtype), native_dtype(acc_dtype),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    host = grad[3:]
+    padded = torch.cat([host, torch.zeros(W * S - host.numel(), dtype=grad_dtype)])
+    want = [torch.zeros(S, dtype=acc_dtype) for _ in range(W)]
+    oracle.scatter_accumulate(want, padded)
+    for r, peer in enumerate(peers):
+        got = peer.cpu()
+        assert_bit_equal(got[guard : guard + S], want[r], f"{grad_dtype}->{acc_dtype} W={W} S={S} rank {r}")
+        assert not torch.signbit(got[guard : guard + S][want[r] == 0]).any()
+        edges = torch.cat([got[:guard], got[guard + S :]]).view(torch.uint8)
+        assert (edges == 0xFF).all(), "bytes outside the slice were written"
+
+
+def test_scatter_store_every_bf16_pattern(make_world):
+    """+0 + g for every bf16 bit pattern g: -0 becomes +0, NaNs stay NaN, all else is g widened."""
+    from odc_amd import ReductionService
+
+    W = 4
+    group = make_world(W, 4 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
+    all_bf16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    red.register("all", (65536 // W,), torch.bfloat16, torch.float32, group)
+    poison(red._registry_peers("all"))
+    red.scatter_accumulate("all", all_bf16.cuda(), group)
+    want = [torch.zeros(65536 // W) for _ in range(W)]
+    oracle.scatter_accumulate(want, all_bf16)
+    for r, acc in enumerate(red.get_peer_accumulations("all")):
+        got, w = acc.cpu(), want[r]
+        nan = torch.isnan(w)
+        assert torch.equal(torch.isnan(got), nan)
+        assert_bit_equal(got[~nan], w[~nan], f"rank {r}")
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_lazy_clear_matches_the_oracle(make_world, seed):
+    """A random minibatch schedule (clears, multi-key launches with repeated and missing keys,
+    reads in between) under lazy clears matches the oracle, which clears eagerly; the
+    accumulations are poisoned behind the service's back after every clear the service skips."""
+    from odc_amd import ReductionService
+
+    rng = random.Random(seed)
+    W = rng.choice([1, 2, 4, 8, 12])
+    grad_dtype, acc_dtype = PAIRS[seed % 6]
+    sizes = {k: rng.choice([1, 63, 512, 4096, 4099, 20_001]) for k in "abcde"}
+    group = make_world(W, 16 << 20)
+    lazy = ReductionService(accumulation_dtype=acc_dtype, lazy_clear=True)
+    g = torch.Generator().manual_seed(seed)
+    want = {k: [torch.zeros(s, dtype=acc_dtype) for _ in range(W)] for k, s in sizes.items()}
+    for k, s in sizes.items():
+        lazy.register(k, (s,), grad_dtype, acc_dtype, group)
+    assert lazy._owed_zero == set(sizes)
+    for minibatch in range(3):
+        lazy.clear_accumulations()
+        for k in sizes:
+            poison(lazy._registry_peers(k))
+            for w in want[k]:
+                w.zero_()
+        for _ in range(rng.randrange(1, 5)):
+            keys = [rng.choice("abcde") for _ in range(rng.randrange(1, 5))]
+            if rng.random() < 0.5:
+                keys = list(dict.fromkeys(keys))  # half of the launches without repeated keys
+            grads = [torch.randn(W * sizes[k], generator=g).to(grad_dtype) for k in keys]
+            lazy.scatter_accumulate_multi(keys, [x.cuda() for x in grads], group)
+            for k, x in zip(keys, grads):
+                oracle.scatter_accumulate(want[k], x)
+            if rng.random() < 0.3:  # a read in the middle of the minibatch
+                k = rng.choice("abcde")
+                for r, acc in enumerate(lazy.get_peer_accumulations(k)):
+                    assert_bit_equal(acc, want[k][r], f"seed {seed}: mid-minibatch read of {k} rank {r}")
+        lazy.sync(group)
+        for k in sizes:  # includes keys no launch touched: they must read as zeros
+            for r, acc in enumerate(lazy.get_peer_accumulations(k)):
+                assert_bit_equal(acc, want[k][r], f"seed {seed}: minibatch {minibatch} key {k} rank {r}")
+        assert not lazy._owed_zero
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_slices_that_tile_the_accumulation_take_the_store_form(make_world, seed):
+    """FSDP2's group layout: the per-parameter slices cover the accumulation exactly, so the
+    first reduce of a minibatch needs no clear; slices with a gap fall back to clear + add."""
+    from odc_amd import ReductionService
+
+    rng = random.Random(50 + seed)
+    W = rng.choice([2, 8, 12])
+    grad_dtype, acc_dtype = PAIRS[seed % 3]
+    sizes = [rng.choice([1, 3, 17, 1000, 4096, 4101, 30_001]) for _ in range(rng.choice([1, 4, 9, 35]))]
+    gap = seed % 2  # odd seeds leave one element uncovered
+    offs, cur = [], 0
+    for i, s in enumerate(sizes):
+        if gap and i == len(sizes) // 2:
+            cur += 1
+        offs.append(cur)
+        cur += s
+    total = cur
+    group = make_world(W, 16 << 20)
+    red = ReductionService(accumulation_dtype=acc_dtype, lazy_clear=True)
+    red.register("g", (total,), grad_dtype, acc_dtype, group)
+    poison(red._registry_peers("g"))
+    g = torch.Generator().manual_seed(seed)
+    want = [torch.zeros(total, dtype=acc_dtype) for _ in range(W)]
+    order = list(range(len(sizes)))
+    for rep in range(2):
+        rng.shuffle(order)  # slice order in the call is free
+        valid = [rng.choice([W * s, rng.randrange(0, W * s + 1)]) for s in sizes]
+        host = [torch.randn(v, generator=g).to(grad_dtype) for v in valid]
+        red.scatter_accumulate_slices("g", [host[i].cuda() for i in order], [offs[i] for i in order],
+                                      [sizes[i] for i in order], group)
+        for hg, o, s in zip(host, offs, sizes):
+            padded = torch.cat([hg, torch.zeros(W * s - hg.numel(), dtype=grad_dtype)])
+            oracle.scatter_accumulate([w[o : o + s] for w in want], padded)
+    for r, acc in enumerate(red.get_peer_accumulations("g")):
+        assert_bit_equal(acc, want[r], f"seed {seed}: W={W} rank {r} sizes {sizes} gap {gap}")
+
+
+def test_clear_stays_eager_under_graph_capture(make_world):
+    """A captured clear must be a kernel in the graph (a lazy clear would be host state only):
+    replaying [clear] alone zeroes the accumulations every time."""
+    from odc_amd import ReductionService
+
+    W, S = 4, 10_001
+    group = make_world(W, 4 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
+    grad = torch.ones(W * S, dtype=torch.bfloat16, device="cuda")
+    red.scatter_accumulate("k", grad, group)
+    red.sync(group)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        red.clear_accumulations()
+    assert not red._owed_zero
+    for replay in range(3):
+        red.scatter_accumulate("k", grad, group)
+        red.scatter_accumulate("k", grad, group)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for acc in red.get_peer_accumulations("k"):
+            assert_bit_equal(acc, torch.zeros(S), f"replay {replay}")
+        red.scatter_accumulate("k", grad, group)
+        for acc in red.get_peer_accumulations("k"):
+            assert_bit_equal(acc, torch.ones(S), f"replay {replay}: one accumulate after the clear")
