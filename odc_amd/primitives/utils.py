@@ -16,6 +16,7 @@ import ctypes
 import logging
 import math
 import os
+import threading
 from functools import reduce
 from typing import List, Optional
 
@@ -416,13 +417,17 @@ def get_local_world_size():
 
 
 stream = None
+_stream_lock = threading.Lock()
 
 
 def get_comm_stream():
-    """One side stream for all primitive launches (``utils.py:205-209``), default priority."""
+    """One side stream for all primitive launches (``utils.py:205-209``), default priority.
+    Callers may come from several host threads (autograd's device thread in backward)."""
     global stream
     if stream is None:
-        stream = torch.cuda.Stream()
+        with _stream_lock:
+            if stream is None:
+                stream = torch.cuda.Stream()
     return stream
 
 

@@ -302,3 +302,48 @@ def test_every_virtual_rank_as_a_client(make_world):
             out = torch.empty(W * S, dtype=torch.bfloat16, device="cuda")
             gather.gather_into_tensor(out, registry.get_symm_buffer("p"), group)
             assert_bit_equal(out, oracle.gather(shards), f"gather as rank {q}")
+
+
+def test_services_called_from_several_host_threads(make_world):
+    """FSDP calls the primitives from the main thread (forward) and from autograd's device thread
+    (backward): concurrent callers, each with keys of its own, must all get exact results."""
+    import threading
+
+    W, S, T, M = 8, 20_003, 4, 12
+    group = make_world(W, 32 << 20)
+    gather, reduction, registry = services()
+    g = torch.Generator().manual_seed(3)
+    shards = {t: [(torch.randn(S, generator=g) * 0.02).bfloat16() for _ in range(W)] for t in range(T)}
+    grads = {t: [(torch.randn(W * S, generator=g) * 1e-3).bfloat16() for _ in range(M)] for t in range(T)}
+    srcs = {t: put_shards(registry, ("p", t), shards[t], group) for t in range(T)}
+    dev_grads = {t: [x.cuda() for x in grads[t]] for t in range(T)}
+    outs = {t: torch.zeros(W * S, dtype=torch.bfloat16, device="cuda") for t in range(T)}
+    for t in range(T):
+        reduction.register(("k", t), (S,), torch.bfloat16, torch.float32, group)
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            torch.cuda.set_device(0)
+            for m in range(M):
+                gather.gather_into_tensor(outs[t], srcs[t], group)
+                reduction.scatter_accumulate(("k", t), dev_grads[t][m], group)
+        except Exception as e:  # noqa: BLE001 - reported on the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(T)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    reduction.sync(group)
+    torch.cuda.synchronize()
+    for t in range(T):
+        assert_bit_equal(outs[t], oracle.gather(shards[t]), f"thread {t}: gather")
+        want = [torch.zeros(S) for _ in range(W)]
+        for m in range(M):
+            oracle.scatter_accumulate(want, grads[t][m])
+        for r, acc in enumerate(reduction.get_peer_accumulations(("k", t))):
+            assert_bit_equal(acc, want[r], f"thread {t}: accumulation of rank {r}")

@@ -86,6 +86,89 @@ def test_arena_offsets_first_fit_and_coalescing():
         a.alloc(1)  # use after finalize
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_arena_random_schedule_against_a_model(seed):
+    """Random allocs and frees checked against a plain first-fit model with 256 B granules: same
+    offsets, no live ranges overlapping, in-use and high-water figures, full coalescing at the end."""
+    import random
+
+    rng = random.Random(seed)
+    cap = 1 << 20
+    a = utils.SymmetricArena(3, cap, backing=False)
+    live = {}  # offset -> rounded size
+    high = 0
+
+    def model_alloc(n):
+        need = max(256, (n + 255) // 256 * 256)
+        cursor = 0
+        for off in sorted(live):
+            if off - cursor >= need:
+                return cursor, need
+            cursor = off + live[off]
+        return (cursor, need) if cap - cursor >= need else (None, need)
+
+    for _ in range(600):
+        if live and rng.random() < 0.45:
+            off = rng.choice(sorted(live))
+            a.free(off)
+            del live[off]
+        else:
+            n = rng.choice([0, 1, 255, 256, 257, 4096, 10_000, 70_000, 200_000])
+            want, need = model_alloc(n)
+            if want is None:
+                with pytest.raises(_native.OdcNativeError) as e:
+                    a.alloc(n)
+                assert e.value.code == _native.ODC_ERR_NOMEM
+            else:
+                assert a.alloc(n) == want
+                live[want] = need
+                high = max(high, want + need)
+        info = a.info()
+        assert info.n_allocations == len(live) and info.bytes_in_use == sum(live.values())
+        assert info.high_water == high
+    for off in list(live):
+        a.free(off)
+    assert a.alloc(cap) == 0  # everything merged back into one block
+    a.destroy()
+
+
+def test_arena_is_safe_to_share_between_host_threads():
+    """The primitives are called from the main thread and from autograd's device thread
+    (FSDP post-backward hooks): concurrent alloc/free/locate-style bookkeeping must keep the
+    allocator consistent. ctypes releases the GIL during the calls."""
+    import random
+    import threading
+
+    a = utils.SymmetricArena(2, 64 << 20, backing=False)
+    errors, held = [], [[] for _ in range(8)]
+
+    def worker(t):
+        rng = random.Random(t)
+        try:
+            for _ in range(2000):
+                if held[t] and rng.random() < 0.5:
+                    a.free(held[t].pop(rng.randrange(len(held[t]))))
+                else:
+                    n = rng.choice([1, 300, 5000, 40_000])
+                    held[t].append((a.alloc(n), n)[0])
+                a.info()
+        except Exception as e:  # noqa: BLE001 - reported below, on the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    offsets = [o for h in held for o in h]
+    assert len(offsets) == len(set(offsets)) == a.info().n_allocations  # nothing handed out twice
+    for o in offsets:
+        a.free(o)
+    assert a.info().bytes_in_use == 0 and a.alloc(64 << 20) == 0
+    a.destroy()
+
+
 def test_sizing_run_for_the_8b_layer():
     """What the bookkeeping-only arena is for: learn the bytes per rank a workload needs."""
     from odc_amd.workloads import llama3_8b_layer_shapes, numel
