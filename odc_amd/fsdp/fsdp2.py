@@ -332,18 +332,26 @@ def foreach_all_gather(fsdp_params, group, async_op, all_gather_copy_in_stream, 
     device_handle = _get_device_handle(device.type)
     out_dtype = fsdp_params[0].param_dtype or layout.dtype
     outs, offsets, numels, dtypes_meta, numels_meta = [], [], [], [], []
-    for fp in fsdp_params:
-        i = layout.index[id(fp)]
-        n = layout.numels[i]
-        fp.init_all_gather_outputs([n], [out_dtype], world_size, device)
-        fp.alloc_all_gather_outputs()  # on the current stream, where torch allocates them too
-        outs.append(fp.all_gather_outputs[0])
-        offsets.append(layout.offsets[i])
-        numels.append(n)
-        dtypes_meta.append([out_dtype])
-        numels_meta.append([n])
+    consumer_stream = device_handle.current_stream()
     all_gather_stream.wait_stream(all_gather_copy_in_stream)
     with device_handle.stream(all_gather_stream):
+        # The unsharded storages are written here, on a stream that runs ahead of the consumer
+        # (implicit prefetch), so they must come from THIS stream's pool: a block of the
+        # consumer's pool may still be in use by kernels queued there. record_stream hands the
+        # block back only after the consumer's work queued up to the free has finished.
+        for fp in fsdp_params:
+            i = layout.index[id(fp)]
+            n = layout.numels[i]
+            fp.init_all_gather_outputs([n], [out_dtype], world_size, device)
+            fp.alloc_all_gather_outputs()
+            out = fp.all_gather_outputs[0]
+            if consumer_stream != all_gather_stream:
+                out.record_stream(consumer_stream)
+            outs.append(out)
+            offsets.append(layout.offsets[i])
+            numels.append(n)
+            dtypes_meta.append([out_dtype])
+            numels_meta.append([n])
         get_gather_service().gather_slices(outs, fsdp_group._odc_symm_buffer, offsets, numels, group)
         all_gather_event = all_gather_stream.record_event()
     placeholder = torch.empty(0, dtype=out_dtype, device=device)
