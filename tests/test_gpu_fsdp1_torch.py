@@ -114,3 +114,21 @@ def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, 
                 off += named[f].numel()
     want_out = copy.deepcopy(reference).bfloat16()(batches[0].bfloat16())
     assert_bit_equal(out, want_out, "forward after the optimizer step")
+
+
+@pytest.mark.parametrize("extra", [
+    ["--world-size", "12", "--layers", "3", "--forward-prefetch"],
+    ["--world-size", "5", "--layers", "2", "--no-backward-prefetch", "--microbatches", "3"],
+])
+def test_transformer_example_trains_bit_exactly(extra):
+    """examples/fsdp1_toy.py: a small transformer under FSDP1 with forward / backward prefetching
+    on and off, at uneven world sizes; every step's flat gradient shards equal the unsharded model's."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    script = Path(__file__).resolve().parent.parent / "examples" / "fsdp1_toy.py"
+    proc = subprocess.run([sys.executable, str(script), "--steps", "3", *extra],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    assert proc.stdout.count("match the unsharded model bit for bit") == 3
