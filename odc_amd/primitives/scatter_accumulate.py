@@ -31,7 +31,7 @@ from odc_amd.primitives.utils import (
     BufferSplitter,
     SymmBufferRegistry,
     comm_stream_section,
-    get_comm_stream,
+    wait_for_launches,
     get_rank,
     get_world,
     group_size,
@@ -326,10 +326,10 @@ class ReductionService:
 
     def sync(self, pg=None):
         """Block until every dispatched add has landed (:734-743: the reference counts tasks
-        across ranks and waits for its watcher; here all adds are on the comm stream)."""
-        get_comm_stream().synchronize()
+        across ranks and waits for its watcher; here it waits for the streams launched on)."""
+        wait_for_launches()
         self.dispatched_tasks = 0
 
     def stop(self):
         if torch.cuda.is_available():
-            get_comm_stream().synchronize()
+            wait_for_launches()

@@ -431,13 +431,36 @@ def get_comm_stream():
     return stream
 
 
+_launch_streams = {}  # cuda_stream handle -> torch stream with launches since the last wait
+
+
+def launch_stream_policy() -> str:
+    """``ODC_COMM_STREAM``: "caller" (default) launches on the caller's current stream;
+    "dedicated" hops to the one comm stream and joins it on both sides, as the reference does."""
+    policy = os.environ.get("ODC_COMM_STREAM", "caller")
+    if policy not in ("caller", "dedicated"):
+        raise ValueError(f"ODC_COMM_STREAM must be 'caller' or 'dedicated', not {policy!r}")
+    return policy
+
+
 @contextlib.contextmanager
 def comm_stream_section():
-    """Run the body's launches on the comm stream, joined with the current stream on both
-    sides (``gather.py:114,176``; ``scatter_accumulate.py:636-640,725-727``). When the caller
-    already runs on the comm stream there is nothing to join."""
-    comm = get_comm_stream()
+    """The stream the body's launches go to.
+
+    The reference hops to its comm stream and joins it with the current stream on both sides
+    (``gather.py:114,176``; ``scatter_accumulate.py:636-640,725-727``), which orders a launch
+    exactly as if it had been issued on the current stream. Here it IS issued on the current
+    stream by default: FSDP already calls the primitives on its own all-gather / reduce-scatter
+    streams, and on this GPU every extra hardware queue with event joins in flight slows the
+    dispatch of all queues (measured on a Llama layer stack: 28.8 -> 22.4 ms per microbatch).
+    ``ODC_COMM_STREAM=dedicated`` restores the hop."""
     current = torch.cuda.current_stream()
+    if launch_stream_policy() == "caller":
+        _launch_streams[current.cuda_stream] = current
+        yield current
+        return
+    comm = get_comm_stream()
+    _launch_streams[comm.cuda_stream] = comm
     if current == comm:
         yield comm
         return
@@ -446,6 +469,13 @@ def comm_stream_section():
         yield comm
     finally:
         current.wait_stream(comm)
+
+
+def wait_for_launches() -> None:
+    """Block the host until every launch issued through ``comm_stream_section`` has finished."""
+    while _launch_streams:
+        _, s = _launch_streams.popitem()
+        s.synchronize()
 
 
 class BufferSplitter:
