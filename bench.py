@@ -33,8 +33,9 @@ MICROBATCHES = 8
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE and
 # WRITE_SIZE runs, scaled by a torch copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("accum", "per-param", 8): 2_181_147_164,
-    ("gather", "per-param", 8): 872_533_161,
+    ("accum", "per-param", 8): 2_181_147_887,
+    ("gather", "per-param", 8): 872_565_155,
+    ("store", "per-param", 8): 1_308_913_261,
 }
 
 
@@ -376,7 +377,8 @@ def main():
         "clear": {"avg_launch_ms": round(c_ms, 5) if c_ms else None,
                   "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},
         "store": {"avg_launch_ms": round(s_ms, 5) if s_ms else None,
-                  "GB/s": round(6 * N / (s_ms * 1e-3) / 1e9, 1) if s_ms else None},
+                  "GB/s": round(6 * N / (s_ms * 1e-3) / 1e9, 1) if s_ms else None,
+                  "traffic": MEASURED_TRAFFIC_BYTES.get(("store", args.layout, W)) if s_ms else None},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 4),
         "cpu_baseline": cpu_baseline,
         "parity_vs_oracle": parity,
