@@ -98,8 +98,14 @@ int64_t* option_slot(const char* name) {
 // ------------------------------------------------------------------------------------------------
 // device side
 // ------------------------------------------------------------------------------------------------
-constexpr int kThreads = 256;  // 4 wavefronts of 64 lanes
-constexpr int kUnroll = 4;     // independent 16 B accesses per lane per stream before the stores
+#ifndef ODC_TILE_THREADS
+#define ODC_TILE_THREADS 256  // 4 wavefronts of 64 lanes
+#endif
+#ifndef ODC_TILE_UNROLL
+#define ODC_TILE_UNROLL 4  // independent 16 B accesses per lane per stream before the stores
+#endif
+constexpr int kThreads = ODC_TILE_THREADS;
+constexpr int kUnroll = ODC_TILE_UNROLL;
 constexpr int kMaxItems = ODC_MAX_ITEMS_PER_LAUNCH;
 constexpr uint32_t kTileVecs = kThreads * kUnroll;      // 16 B vectors per tile
 constexpr uint32_t kTileBytes = kTileVecs * 16;         // gather / clear: 16 KiB of destination
