@@ -305,6 +305,25 @@ def main():
         elapsed = time.perf_counter() - t0
         if os.environ.get("ODC_BENCH_DEBUG"):
             print("host ms per step:", [round(x * 1e3, 3) for x in host_step], file=sys.stderr)
+        # the same steps once more in the other clear mode (no events): a secondary figure
+        other = None
+        if args.steps >= MICROBATCHES:
+            reduction.lazy_clear = not args.lazy_clear
+            for i in range(MICROBATCHES):
+                step(i, record=False)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for i in range(args.steps):
+                step(i, record=False)
+            torch.cuda.synchronize()
+            other_elapsed = time.perf_counter() - t1
+            stores = len(range(0, args.steps, MICROBATCHES)) if reduction.lazy_clear else 0
+            other_bytes = 14 * N * args.steps - 4 * N * stores
+            other = {"clear": "lazy (store on the first microbatch)" if reduction.lazy_clear else "eager",
+                     "value": round(other_bytes / other_elapsed / 1e9, 1), "unit": "GB/s",
+                     "bytes_per_step": round(other_bytes / args.steps),
+                     "minibatch_ms": round(other_elapsed / args.steps * MICROBATCHES * 1e3, 4)}
+            reduction.lazy_clear = args.lazy_clear
     gc.enable()
 
     if args.calibrate:
@@ -380,6 +399,7 @@ def main():
                   "GB/s": round(6 * N / (s_ms * 1e-3) / 1e9, 1) if s_ms else None,
                   "traffic": MEASURED_TRAFFIC_BYTES.get(("store", args.layout, W)) if s_ms else None},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 4),
+        "other_clear_mode": other,
         "cpu_baseline": cpu_baseline,
         "parity_vs_oracle": parity,
     }
