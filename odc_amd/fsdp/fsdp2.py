@@ -413,6 +413,12 @@ def foreach_reduce(fsdp_params, unsharded_grads, reduce_scatter_group, reduce_sc
             accumulation_numel=layout.total, accumulation_dtype=reduce_dtype,
         )
         reduce_scatter_event = reduce_scatter_stream.record_event()
+        # parameters that got a gradient in some microbatch of this minibatch: only they are
+        # handed one at the optimizer step (frozen or unused parameters keep grad = None)
+        touched = getattr(fsdp_group, "_odc_params_with_grad", None)
+        if touched is None:
+            touched = fsdp_group._odc_params_with_grad = set()
+        touched.update(id(fp) for fp in fsdp_params)
         fsdp_group._odc_reduce_context = dict(
             reduce_scatter_group=reduce_scatter_group, reduce_scatter_stream=reduce_scatter_stream,
             orig_dtype=orig_dtype, reduce_dtype=reduce_dtype, device=device,
@@ -438,6 +444,7 @@ def update_gradients(fsdp_param_group) -> None:
     if ctx is None:
         return  # no microbatch ran through this group in this minibatch (fsdp2.py:797-801)
     del fsdp_param_group._odc_reduce_context
+    touched = fsdp_param_group.__dict__.pop("_odc_params_with_grad", None)
     layout = _group_layout(fsdp_param_group)
     rs_group = ctx["reduce_scatter_group"]
     _pre, postdivide_factor, reduce_scatter_op, _ar_op = _get_gradient_divide_factors(
@@ -461,6 +468,8 @@ def update_gradients(fsdp_param_group) -> None:
         (reduce_output,) = scatter.publish([key], out_dtype=orig_dtype, divisor=divisor)
     base = reduce_output.storage_offset()
     for fp, off in zip(fsdp_param_group.fsdp_params, layout.offsets):
+        if touched is not None and id(fp) not in touched:
+            continue
         new_sharded_grad = torch.as_strided(
             reduce_output, size=fp.sharded_size, stride=fp.contiguous_sharded_stride,
             storage_offset=base + off,

@@ -160,3 +160,57 @@ def test_transformer_example_trains_bit_exactly(extra):
                           capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert proc.stdout.count("match the unsharded model bit for bit") == 4
+
+
+def test_frozen_and_unused_parameters_get_no_gradient(make_world, fake_process_group):
+    """A group whose gradients cover only part of its accumulation (one parameter frozen, one
+    module never called): the rest is reduced exactly, the two keep ``grad is None`` as under
+    torch's own FSDP, and the partial cover takes the clear + accumulate route of lazy clears."""
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.fsdp import fully_shard
+
+    from odc_amd.fsdp import fsdp2
+
+    W = 4
+    fake_process_group(W)
+    mesh = init_device_mesh("cuda", (W,))
+    make_world(W, 64 << 20)
+    fsdp2.patch_fsdp2()
+    torch.manual_seed(0)
+    model = Toy().cuda()
+    model.spare = nn.Linear(7, 5).cuda()  # never used in forward
+    model.layers[1].up.bias.requires_grad_(False)
+    reference = copy.deepcopy(model)
+    full_params = {name: p.detach().clone() for name, p in reference.named_parameters()}
+    for layer in model.layers:
+        fully_shard(layer, mesh=mesh)
+    fully_shard(model, mesh=mesh)
+    for layer in model.layers:
+        fsdp2.patch_lazy_init(layer)
+    fsdp2.patch_lazy_init(model)
+    fully_shard.state(model)._lazy_init()
+    for module in [*model.layers, model]:
+        fsdp2.fill_peer_shards(module, full_params)
+
+    g = torch.Generator().manual_seed(5)
+    batches = [torch.randn(16, 32, generator=g).cuda() for _ in range(2)]
+    for minibatch in range(2):  # the second one starts from accumulations that hold old sums
+        fsdp2.pre_minibatch_start(model)
+        want = {name: torch.zeros(p.numel()) for name, p in full_params.items()}
+        for x in batches:
+            model(x).pow(2).mean().backward()
+            reference.zero_grad(set_to_none=True)
+            reference(x).pow(2).mean().backward()
+            for name, p in reference.named_parameters():
+                if p.grad is not None:
+                    want[name].add_(p.grad.detach().cpu().reshape(-1))
+        fsdp2.pre_optimizer_step(model)
+        for name, p in model.named_parameters():
+            if name.startswith("spare.") or name == "layers.1.up.bias":
+                assert p.grad is None, name
+                continue
+            rows = math.ceil(full_params[name].shape[0] / W)
+            rest = full_params[name][0].numel() if full_params[name].dim() > 1 else 1
+            expect = oracle.fsdp2_average(want[name][: rows * rest].clone(), W).view(p._local_tensor.shape)
+            assert_bit_equal(p.grad._local_tensor, expect, f"minibatch {minibatch}: sharded gradient of {name}")
+        model.zero_grad(set_to_none=True)
