@@ -282,9 +282,9 @@ def main():
         del host_params, host_grads, host_outs, host_accs, host_shards
 
     # ---- timed region -----------------------------------------------------------------------
-    # The services launch on the comm stream (as the reference does). Making it the current
-    # stream here removes the stream joins from between the event pairs, so that each pair
-    # brackets exactly one kernel.
+    # The services launch on the caller's current stream. The timed loop runs on a side stream
+    # of its own (not torch's default stream), and the events are recorded on that same stream,
+    # so that each pair of events brackets exactly one kernel.
     # A full Python garbage collection (tens of ms with torch imported) landing inside the timed
     # loop would stall the launches while an event pair is open: collect now, then keep the
     # collector off until the loop is done.
