@@ -61,6 +61,9 @@ def get_shard(tensor: torch.Tensor, rank: int, world_size: int):
     return sharded_in_symm, numel_to_pad
 
 
+custom_get_shard = get_shard  # the reference's name for it (fsdp1.py:239)
+
+
 def all_gather_flat_param(padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=None):
     """Gather the padded flat parameter. The shards stay in their own dtype (a peer may not have
     produced a low-precision copy yet: that is why the reference gathers in the shard dtype into

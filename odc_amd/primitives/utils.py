@@ -236,7 +236,53 @@ def finalize_distributed():
             SymmBufferRegistry._instance._forget()
         _world.arena.destroy()
         _world = None
+    _bare_allocations.clear()
     stream = None
+
+
+# symmetric allocations made through the reference's bare helpers: local data_ptr -> (offset, shape, dtype)
+_bare_allocations = {}
+
+
+def nvshmem_create_tensor(shape, dtype) -> torch.Tensor:
+    """A symmetric tensor outside the registry (``utils.py:53-57``): the calling rank's view of
+    a fresh arena allocation that exists, at the same offset, in every rank region."""
+    world = get_world()
+    shape = tuple(shape) if not isinstance(shape, int) else (shape,)
+    offset = world.arena.alloc(max(1, math.prod(shape)) * dtype.itemsize)
+    tensor = world.arena.view(get_rank(), offset, shape, dtype)
+    _bare_allocations[tensor.data_ptr()] = (offset, shape, dtype)
+    return tensor
+
+
+def get_same_node_tensors(tensor, rank, local_world_size) -> List[torch.Tensor]:
+    """The views of ``tensor``'s symmetric allocation on every rank of ``rank``'s node
+    (``utils.py:60-75``); the entry for ``rank`` is ``tensor`` itself. ``tensor`` is any
+    symmetric tensor of any rank: made by ``nvshmem_create_tensor`` or by the registry."""
+    world = get_world()
+    _owner, offset, inner = world.arena.locate(tensor.data_ptr())
+    first = rank - rank % local_world_size
+    return [
+        tensor if peer == rank else world.arena.view(peer, offset + inner, tuple(tensor.shape), tensor.dtype)
+        for peer in range(first, first + local_world_size)
+    ]
+
+
+def nvshmem_free_tensor_sync(tensor) -> None:
+    """Free a tensor made by ``nvshmem_create_tensor`` (``utils.py:78-81``), after the device has
+    finished with it. The tensor and its peers dangle afterwards."""
+    entry = _bare_allocations.pop(tensor.data_ptr(), None)
+    if entry is None:
+        raise ValueError("tensor was not made by nvshmem_create_tensor (or was freed already)")
+    torch.cuda.synchronize()
+    get_world().arena.free(entry[0])
+
+
+def get_local_world_pg(pg):
+    """The group of the calling rank's node (``utils.py:178-192``). All W virtual ranks share
+    one GPU, hence one node: the group itself."""
+    assert group_size(pg) == get_world().world_size, "the group must span the virtual world"
+    return pg
 
 
 def get_rank() -> int:

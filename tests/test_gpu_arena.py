@@ -127,3 +127,41 @@ def test_plain_c_client_of_the_abi():
     proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "abi_check ok" in proc.stdout
+
+
+def test_reference_named_symmetric_tensor_helpers(make_world):
+    """nvshmem_create_tensor / get_same_node_tensors / nvshmem_free_tensor_sync / get_local_world_pg
+    (odc/primitives/utils.py:53-81,178-192) on the arena: peers alias one offset in W regions."""
+    import torch
+
+    from odc_amd import virtual_rank
+    from odc_amd.primitives import utils
+
+    W = 4
+    group = make_world(W, 1 << 20)
+    with virtual_rank(2):
+        mine = utils.nvshmem_create_tensor((3, 5), torch.float32)
+        peers = utils.get_same_node_tensors(mine, 2, W)
+    assert len(peers) == W and peers[2] is mine
+    arena = utils.get_world().arena
+    offsets = set()
+    for r, t in enumerate(peers):
+        t.fill_(float(r))
+        rank, off, inner = arena.locate(t.data_ptr())
+        assert rank == r and inner == 0 and tuple(t.shape) == (3, 5)
+        offsets.add(off)
+    assert len(offsets) == 1  # symmetric: the same offset in every rank region
+    for r, t in enumerate(peers):
+        assert (t == float(r)).all()
+    # a registry buffer works as the handle too, from any rank's view
+    reg = utils.SymmBufferRegistry.get_instance()
+    buf = reg.allocate_symm_buffer("x", (8,), torch.int32)
+    views = utils.get_same_node_tensors(buf, utils.get_rank(), W)
+    for r, (a, b) in enumerate(zip(views, reg.peer_tensors["x"])):
+        assert a.data_ptr() == b.data_ptr(), r
+    assert utils.get_local_world_pg(group) is group
+    before = arena.info().n_allocations
+    utils.nvshmem_free_tensor_sync(mine)
+    assert arena.info().n_allocations == before - 1
+    with pytest.raises(ValueError):
+        utils.nvshmem_free_tensor_sync(mine)
