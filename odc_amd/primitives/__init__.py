@@ -11,6 +11,7 @@ _native.load()  # raises ImportError when the HIP library has not been built
 
 from odc_amd.primitives.gather import GatherService  # noqa: E402
 from odc_amd.primitives.scatter_accumulate import ReductionService  # noqa: E402
+from odc_amd.primitives.tensor_ipc import get_ipc_handle, reconstruct_tensor  # noqa: E402
 from odc_amd.primitives.utils import (  # noqa: E402
     BufferSplitter,
     SymmBufferRegistry,
@@ -39,4 +40,6 @@ __all__ = [
     "get_world_size",
     "set_rank",
     "virtual_rank",
+    "get_ipc_handle",
+    "reconstruct_tensor",
 ]

@@ -165,3 +165,37 @@ def test_reference_named_symmetric_tensor_helpers(make_world):
     assert arena.info().n_allocations == before - 1
     with pytest.raises(ValueError):
         utils.nvshmem_free_tensor_sync(mine)
+
+
+def test_tensor_ipc_handles_round_trip(make_world):
+    """get_ipc_handle / reconstruct_tensor (csrc/tensor_ipc/tensor_ipc.cu:24-57) inside one
+    process: 72-byte handles of whole buffers and of inner views, for every rank."""
+    import torch
+
+    from odc_amd import SymmBufferRegistry, virtual_rank
+    from odc_amd.primitives import get_ipc_handle, reconstruct_tensor
+
+    W = 3
+    make_world(W, 1 << 20)
+    reg = SymmBufferRegistry.get_instance()
+    reg.allocate_symm_buffer("acc", (1000,), torch.float32)
+    for r, peer in enumerate(reg.peer_tensors["acc"]):
+        peer.copy_(torch.arange(1000, dtype=torch.float32) + 1000 * r)
+    for r in range(W):
+        with virtual_rank(r):
+            local = reg.get_symm_buffer("acc")
+        handle = get_ipc_handle(local)
+        assert isinstance(handle, bytes) and len(handle) == 72
+        again = reconstruct_tensor(handle, (1000,), torch.float32)
+        assert again.data_ptr() == local.data_ptr() and torch.equal(again, local)
+        inner = get_ipc_handle(local[100:])  # the reference adds the pointer's offset to the handle
+        part = reconstruct_tensor(inner, (10, 5), torch.float32)
+        assert torch.equal(part.reshape(-1), local[100:150])
+        as_bytes = reconstruct_tensor(inner, (8,), torch.uint8)
+        assert torch.equal(as_bytes, local[100:102].view(torch.uint8))
+    with pytest.raises(ValueError):
+        reconstruct_tensor(b"\0" * 72, (1,), torch.float32)
+    with pytest.raises(ValueError):
+        reconstruct_tensor(handle[:10], (1,), torch.float32)
+    with pytest.raises(Exception):
+        get_ipc_handle(torch.zeros(4, device="cuda"))  # not in the arena
