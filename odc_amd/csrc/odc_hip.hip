@@ -248,25 +248,29 @@ __device__ __forceinline__ SegShape seg_shape(uintptr_t written_addr, uint64_t n
 // head and the tail. Kept out of line so that the streaming loop stays tight.
 __device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t* s, uint32_t chunk,
                                                        SegShape g) {
+  // Every load of the tile is issued before its first store (a lone resident workgroup would
+  // otherwise pay one memory round trip per step).
   const uint32_t tid = threadIdx.x;
   const uint64_t v0 = (uint64_t)chunk * kTileVecs;
-  if (v0 < g.nvec && v0 + kTileVecs > g.nvec) {
-    const uint32_t left = (uint32_t)(g.nvec - v0);
-    const uint8_t* sb = s + g.head + v0 * 16;
-    u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
-    u32x4 v[kUnroll];
+  const bool run = v0 < g.nvec && v0 + kTileVecs > g.nvec;
+  const uint32_t left = run ? (uint32_t)(g.nvec - v0) : 0u;
+  const uint8_t* sb = s + g.head + v0 * 16;
+  u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
+  const bool do_head = chunk == 0 && tid < g.head;
+  const bool do_tail = chunk == g.last && tid < g.tail;
+  const uint64_t tail_at = g.head + g.nvec * 16 + tid;
+  u32x4 v[kUnroll];
+  uint8_t head_byte = 0, tail_byte = 0;
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (u * kThreads + tid < left) v[u] = load_stream<u32x4>(sb + (size_t)(u * kThreads + tid) * 16);
+  for (int u = 0; u < kUnroll; ++u)
+    if (u * kThreads + tid < left) v[u] = load_stream<u32x4>(sb + (size_t)(u * kThreads + tid) * 16);
+  if (do_head) head_byte = s[tid];
+  if (do_tail) tail_byte = s[tail_at];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (u * kThreads + tid < left) __builtin_nontemporal_store(v[u], db + u * kThreads + tid);
-  }
-  if (chunk == 0 && tid < g.head) d[tid] = s[tid];
-  if (chunk == g.last && tid < g.tail) {
-    const uint64_t o = g.head + g.nvec * 16 + tid;
-    d[o] = s[o];
-  }
+  for (int u = 0; u < kUnroll; ++u)
+    if (u * kThreads + tid < left) __builtin_nontemporal_store(v[u], db + u * kThreads + tid);
+  if (do_head) d[tid] = head_byte;
+  if (do_tail) d[tail_at] = tail_byte;
 }
 
 // True when tile `chunk` of a segment has anything besides whole runs of vectors to do.
@@ -409,66 +413,75 @@ template <> struct Quad<f16_tag> {
 
 // kStore: the accumulation is taken to hold +0 and is not read (acc = +0 + g, the value a clear
 // followed by an accumulate leaves: -0 gradients still become +0).
-template <class G, class A, bool kStore>
-__device__ __forceinline__ void accum_one(uint8_t* acc, const uint8_t* grad, uint64_t gi,
-                                          uint64_t grad_elems, uint64_t i) {
-  typedef typename Codec<A>::raw_t araw_t;
-  typedef typename Codec<G>::raw_t graw_t;
-  araw_t* a = reinterpret_cast<araw_t*>(acc) + i;
-  float g = 0.0f;  // padding reads as +0 and is still added (so -0 + +0 -> +0, as F.pad + add_)
-  if (gi < grad_elems) g = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi]);
-  float before = 0.0f;
-  if constexpr (!kStore) before = Codec<A>::widen(*a);
-  *a = Codec<A>::narrow(before + g);
-}
-
-// One quad (4 elements) of a tile that is partial, crosses the end of the valid gradient, or
-// lies in the zero padding. acc points at the quad, gi is its first element's gradient index.
-template <class G, class A, bool kStore>
-__device__ __forceinline__ void accum_quad_guarded(uint8_t* acc, const uint8_t* grad, uint64_t gi,
-                                                   uint64_t grad_elems) {
-  typedef typename Quad<G>::vec_t gvec_t;
-  typedef typename Quad<A>::vec_t avec_t;
-  avec_t* ap = reinterpret_cast<avec_t*>(acc);
-  float gf[4] = {0.0f, 0.0f, 0.0f, 0.0f}, af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (gi + 4 <= grad_elems) {
-    Quad<G>::widen(load_stream<gvec_t>(grad + gi * Codec<G>::kBytes), gf);
-  } else {
-    typedef typename Codec<G>::raw_t graw_t;
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      if (gi + k < grad_elems) gf[k] = Codec<G>::widen(reinterpret_cast<const graw_t*>(grad)[gi + k]);
-  }
-  if constexpr (!kStore) Quad<A>::widen(__builtin_nontemporal_load(ap), af);
-#pragma unroll
-  for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
-  __builtin_nontemporal_store(Quad<A>::narrow(af), ap);
-}
-
+//
 // The parts of a tile that are not whole runs of valid quads: a partial last run, a run that
 // crosses the end of the valid gradient or lies in the zero padding, the head and the tail.
+// Gradient elements at index >= grad_elems read as +0 and are still added (so an accumulation
+// holding -0 becomes +0, as F.pad followed by add_ leaves it). Two phases, every load of the tile
+// before its first store: a lone resident workgroup would otherwise pay one memory round trip
+// per quad.
 template <class G, class A, bool kStore>
 __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_t* grad, uint64_t g_seg,
                                                       uint64_t grad_elems, uint32_t chunk, SegShape g,
                                                       bool body) {
-  constexpr uint32_t kAB = Codec<A>::kBytes;
+  typedef typename Quad<G>::vec_t gvec_t;
+  typedef typename Quad<A>::vec_t avec_t;
+  typedef typename Codec<G>::raw_t graw_t;
+  typedef typename Codec<A>::raw_t araw_t;
+  constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
   const uint32_t tid = threadIdx.x;
   const uint64_t q0 = (uint64_t)chunk * kTileVecs;
-  if (body && q0 < g.nvec) {
-    const uint64_t left = g.nvec - q0;
-    const uint64_t e0 = g.head + q0 * 4;
+  const uint64_t left = body && q0 < g.nvec ? g.nvec - q0 : 0;
+  const uint64_t e0 = g.head + q0 * 4;
+  avec_t* ap = reinterpret_cast<avec_t*>(acc + e0 * kAB);
+  const graw_t* gs = reinterpret_cast<const graw_t*>(grad);
+  araw_t* as = reinterpret_cast<araw_t*>(acc);
+  const bool do_head = chunk == 0 && tid < g.head;
+  const bool do_tail = chunk == g.last && tid < g.tail;
+  const uint64_t tail_at = g.head + g.nvec * 4 + tid;
+
+  float gf[kUnroll][4];
+  avec_t araw[kUnroll];
+  float head_g = 0.0f, head_a = 0.0f, tail_g = 0.0f, tail_a = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const uint32_t q = u * kThreads + tid;
-      if (q < left)
-        accum_quad_guarded<G, A, kStore>(acc + (e0 + (uint64_t)q * 4) * kAB, grad, g_seg + e0 + (uint64_t)q * 4, grad_elems);
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t q = u * kThreads + tid;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) gf[u][k] = 0.0f;
+    if (q < left) {
+      const uint64_t gi = g_seg + e0 + (uint64_t)q * 4;
+      if (gi + 4 <= grad_elems) {
+        Quad<G>::widen(load_stream<gvec_t>(grad + gi * kGB), gf[u]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (gi + k < grad_elems) gf[u][k] = Codec<G>::widen(gs[gi + k]);
+      }
+      if constexpr (!kStore) araw[u] = __builtin_nontemporal_load(ap + q);
     }
   }
-  if (chunk == 0 && tid < g.head) accum_one<G, A, kStore>(acc, grad, g_seg + tid, grad_elems, tid);
-  if (chunk == g.last && tid < g.tail) {
-    const uint64_t i = g.head + g.nvec * 4 + tid;
-    accum_one<G, A, kStore>(acc, grad, g_seg + i, grad_elems, i);
+  if (do_head) {
+    if (g_seg + tid < grad_elems) head_g = Codec<G>::widen(gs[g_seg + tid]);
+    if constexpr (!kStore) head_a = Codec<A>::widen(as[tid]);
   }
+  if (do_tail) {
+    if (g_seg + tail_at < grad_elems) tail_g = Codec<G>::widen(gs[g_seg + tail_at]);
+    if constexpr (!kStore) tail_a = Codec<A>::widen(as[tail_at]);
+  }
+
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t q = u * kThreads + tid;
+    if (q < left) {
+      float af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (!kStore) Quad<A>::widen(araw[u], af);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[u][k];
+      __builtin_nontemporal_store(Quad<A>::narrow(af), ap + q);
+    }
+  }
+  if (do_head) as[tid] = Codec<A>::narrow(head_a + head_g);
+  if (do_tail) as[tail_at] = Codec<A>::narrow(tail_a + tail_g);
 }
 
 template <class G, class A, bool kStore>
@@ -518,36 +531,44 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
 // dst[r*S + i] = narrow_D(widen_S(region_r[off + i])): the gather of shards kept in one dtype
 // (fp32 master copies) into a full parameter of another (bf16), in one pass.
 template <class S, class D>
-__device__ __forceinline__ void cast_one(uint8_t* d, const uint8_t* s, uint64_t i) {
-  typedef typename Codec<S>::raw_t sraw_t;
-  typedef typename Codec<D>::raw_t draw_t;
-  reinterpret_cast<draw_t*>(d)[i] = Codec<D>::narrow(Codec<S>::widen(reinterpret_cast<const sraw_t*>(s)[i]));
-}
-
-template <class S, class D>
 __device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* s, uint32_t chunk, SegShape g) {
   typedef typename Quad<S>::vec_t svec_t;
   typedef typename Quad<D>::vec_t dvec_t;
+  typedef typename Codec<S>::raw_t sraw_t;
+  typedef typename Codec<D>::raw_t draw_t;
   constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
   const uint32_t tid = threadIdx.x;
   const uint64_t q0 = (uint64_t)chunk * kTileVecs;
-  if (q0 < g.nvec && q0 + kTileVecs > g.nvec) {
-    const uint64_t left = g.nvec - q0;
-    const uint64_t e0 = g.head + q0 * 4;
-    const uint8_t* sb = s + e0 * kSB;
-    dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB);
+  const uint64_t left = q0 < g.nvec && q0 + kTileVecs > g.nvec ? g.nvec - q0 : 0;
+  const uint64_t e0 = g.head + q0 * 4;
+  const uint8_t* sb = s + e0 * kSB;
+  dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB);
+  const sraw_t* ss = reinterpret_cast<const sraw_t*>(s);
+  draw_t* ds = reinterpret_cast<draw_t*>(d);
+  const bool do_head = chunk == 0 && tid < g.head;
+  const bool do_tail = chunk == g.last && tid < g.tail;
+  const uint64_t tail_at = g.head + g.nvec * 4 + tid;
+  // every load of the tile before its first store
+  svec_t raw[kUnroll];
+  sraw_t head_raw = 0, tail_raw = 0;
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const uint32_t q = u * kThreads + tid;
-      if (q < left) {
-        float f[4];
-        Quad<S>::widen(load_stream<svec_t>(sb + (size_t)q * sizeof(svec_t)), f);
-        __builtin_nontemporal_store(Quad<D>::narrow(f), dp + q);
-      }
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t q = u * kThreads + tid;
+    if (q < left) raw[u] = load_stream<svec_t>(sb + (size_t)q * sizeof(svec_t));
+  }
+  if (do_head) head_raw = ss[tid];
+  if (do_tail) tail_raw = ss[tail_at];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t q = u * kThreads + tid;
+    if (q < left) {
+      float f[4];
+      Quad<S>::widen(raw[u], f);
+      __builtin_nontemporal_store(Quad<D>::narrow(f), dp + q);
     }
   }
-  if (chunk == 0 && tid < g.head) cast_one<S, D>(d, s, tid);
-  if (chunk == g.last && tid < g.tail) cast_one<S, D>(d, s, g.head + g.nvec * 4 + tid);
+  if (do_head) ds[tid] = Codec<D>::narrow(Codec<S>::widen(head_raw));
+  if (do_tail) ds[tail_at] = Codec<D>::narrow(Codec<S>::widen(tail_raw));
 }
 
 template <class S, class D>
@@ -619,14 +640,23 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
         if (out) __builtin_nontemporal_store(Quad<O>::narrow(f), op + u * kThreads);
       }
     } else {
+      // element by element (a partial or unaligned tile), all loads before the first store
+      constexpr int kPerLane = kTileElems / kThreads;
       const uint32_t n = left < kTileElems ? (uint32_t)left : kTileElems;
-      for (uint32_t i = tid; i < n; i += kThreads) {
-        araw_t raw = acc[i];
-        if (launch.divide) {
-          raw = Codec<A>::narrow(Codec<A>::widen(raw) / launch.divisor);
-          acc[i] = raw;
+      araw_t raw[kPerLane];
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j)
+        if (j * kThreads + tid < n) raw[j] = acc[j * kThreads + tid];
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) {
+        const uint32_t i = j * kThreads + tid;
+        if (i < n) {
+          if (launch.divide) {
+            raw[j] = Codec<A>::narrow(Codec<A>::widen(raw[j]) / launch.divisor);
+            acc[i] = raw[j];
+          }
+          if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw[j]));
         }
-        if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw));
       }
     }
   }
@@ -1199,10 +1229,16 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
         });
     if (n < 0) return n;
     if (n == 0) continue;
+    // The persistent shape (one workgroup per CU) streams fastest, but only while every rank's
+    // chunk of the gradient and of the accumulation starts on a 128 B line: with nothing else
+    // resident to cover for it, a workgroup whose wavefronts straddle lines, or that meets heads,
+    // tails and padding, falls behind (measured: -7 % on 16 B aligned uneven shards, against
+    // +1..3 % on line-aligned ones). Everything else runs one workgroup per tile.
     bool ragged = false;
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
-      ragged |= (L.acc_off[k] & 15u) != 0 || (L.seg_elems[k] & 3u) != 0 ||
-                ((uintptr_t)L.grad[k] & (4u * gb - 1)) != 0 || L.grad_elems[k] != L.seg_elems[k] * a->world;
+      ragged |= (L.acc_off[k] & 127u) != 0 || ((L.seg_elems[k] * ab) & 127u) != 0 ||
+                ((L.seg_elems[k] * gb) & 127u) != 0 || ((uintptr_t)L.grad[k] & 127u) != 0 ||
+                L.grad_elems[k] != L.seg_elems[k] * a->world;
     const uint32_t grid =
         grid_for(a, store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
     const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
