@@ -110,7 +110,7 @@ int odc_arena_locate(const odc_arena* arena, const void* ptr, uint32_t* rank,
  * byte copy, so any element type. first_rank rotates the order in which rank regions are walked
  * (gather.py:122); it never changes the result. dst must not overlap the arena ranges read.
  * ---------------------------------------------------------------------------------------- */
-#define ODC_MAX_ITEMS_PER_LAUNCH 32
+#define ODC_MAX_ITEMS_PER_LAUNCH 64
 
 typedef struct odc_gather_item {
   void* dst;             /* device pointer to W*shard_bytes writable bytes */

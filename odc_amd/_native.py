@@ -43,7 +43,7 @@ EXPORTED_SYMBOLS = (
 )
 
 ABI_VERSION = 1
-MAX_ITEMS_PER_LAUNCH = 32
+MAX_ITEMS_PER_LAUNCH = 64
 
 ODC_OK = 0
 ODC_ERR_INVALID = -1

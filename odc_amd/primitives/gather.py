@@ -43,7 +43,7 @@ class GatherService:
     def gather_into_tensors(
         self, output_tensors: Sequence[Tensor], input_tensors: Sequence[Tensor], pg
     ) -> None:
-        """Multi-tensor form: every (output, input) pair of the lists in ONE launch (per 32
+        """Multi-tensor form: every (output, input) pair of the lists in ONE launch (per 64
         pairs). Equivalent to calling ``gather_into_tensor`` pair by pair. When the outputs'
         dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)

@@ -141,7 +141,7 @@ class ReductionService:
     def scatter_accumulate_multi(
         self, keys: Sequence, input_tensors: Sequence[torch.Tensor], pg, valid_numels=None
     ) -> None:
-        """Multi-tensor form: all (key, gradient) pairs in ONE launch (per 32 pairs).
+        """Multi-tensor form: all (key, gradient) pairs in ONE launch (per 64 pairs).
 
         ``valid_numels[i]``, when given, says that only the first so many elements of the
         padded gradient i exist at ``input_tensors[i]``; the rest read as +0 (the ``F.pad`` of

@@ -95,7 +95,7 @@ def test_config3_uneven_padded_w12(make_world):
                 registry.update_symm_buffer(i, oracle.fsdp1_get_shard(p, r, W).cuda())
         locals_.append(registry.get_symm_buffer(i))
     outs = [torch.full((W * s,), float("nan"), dtype=torch.bfloat16, device="cuda") for s in shard]
-    gather.gather_into_tensors(outs, locals_, group)  # 40 items -> 2 launches of <= 32
+    gather.gather_into_tensors(outs, locals_, group)  # 40 items, one launch
     for i, (o, p) in enumerate(zip(outs, host_params)):
         want = oracle.gather([oracle.fsdp1_get_shard(p, r, W) for r in range(W)])
         assert_bit_equal(o, want, f"param {i} (numel {numels[i]})")
