@@ -45,8 +45,10 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--world-size", type=int, default=8, help="virtual ranks W")
-    ap.add_argument("--workload", choices=["layer", "model"], default="layer",
-                    help="layer: one Llama-3-8B decoder layer (the headline); model: the full 8.03 G "
+    ap.add_argument("--workload", choices=["layer", "uneven", "model"], default="layer",
+                    help="layer: one Llama-3-8B decoder layer (the headline); uneven: 40 flat parameters of "
+                         "log-uniform size, none divisible by W (run it with --world-size 12): shards are "
+                         "zero padded and the gradients end before the padding; model: the full 8.03 G "
                          "parameter model swept unit by unit (needs ~85 GB of HBM; no oracle pass)")
     ap.add_argument("--layout", choices=["per-param", "flat"], default="per-param",
                     help="9 per-parameter shards in one multi-tensor launch, or one flat shard")
@@ -164,7 +166,7 @@ def main():
     import odc_amd
     from odc_amd import _native
     from odc_amd.primitives.utils import get_comm_stream
-    from odc_amd.workloads import llama3_8b_layer_shapes, numel
+    from odc_amd.workloads import llama3_8b_layer_shapes, numel, shard_numel, uneven_flat_numels
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
@@ -176,8 +178,13 @@ def main():
     shapes = llama3_8b_layer_shapes()
     if args.layout == "flat":
         shapes = [("flat", (sum(numel(s) for _, s in shapes),))]
-    numels = [numel(s) for _, s in shapes]
-    assert all(n % W == 0 for n in numels)
+    valid = [numel(s) for _, s in shapes]  # elements that exist; the rest of W * shard is padding
+    if args.workload == "uneven":
+        valid = uneven_flat_numels(40, W)
+        shapes = [(f"flat{i}", (n,)) for i, n in enumerate(valid)]
+    numels = [W * shard_numel(n, W) for n in valid]  # padded: what the kernels move
+    padded = numels != valid
+    assert padded == (args.workload == "uneven")
     N = sum(numels)
     per_rank = sum((n // W) * 6 + 512 for n in numels) + (1 << 20)
     group = odc_amd.init_nvshmem(world_size=W, symmetric_size=per_rank)
@@ -188,7 +195,9 @@ def main():
     # synthetic data, generated on the device and mirrored to the host for the oracle
     dev_gen = torch.Generator(device="cuda").manual_seed(0)
     params = [(torch.randn(n, generator=dev_gen, device="cuda") * 0.02).bfloat16() for n in numels]
-    grads = [[(torch.randn(n, generator=dev_gen, device="cuda") * 1e-3).bfloat16() for n in numels]
+    for p, v in zip(params, valid):
+        p[v:] = 0  # the zero padding of the last shards (odc/fsdp/fsdp1.py:239-247)
+    grads = [[(torch.randn(v, generator=dev_gen, device="cuda") * 1e-3).bfloat16() for v in valid]
              for _ in range(MICROBATCHES)]
     keys = [name for name, _ in shapes]
     shard_locals = []
@@ -222,7 +231,7 @@ def main():
         gather.gather_into_tensors(outs, shard_locals, group)
         if record:
             mark("gather")
-        reduction.scatter_accumulate_multi(keys, grads[m], group)
+        reduction.scatter_accumulate_multi(keys, grads[m], group, valid_numels=valid if padded else None)
         if record:
             mark("store" if m == 0 and args.lazy_clear else "accum")
 
@@ -236,7 +245,8 @@ def main():
             step(i, record=False)
         reduction.sync(group)
         host_params = [p.cpu() for p in params]
-        host_grads = [[g.cpu() for g in mb] for mb in grads]
+        host_grads = [[torch.cat([g.cpu(), torch.zeros(n - g.numel(), dtype=g.dtype)]) if padded else g.cpu()
+                       for g, n in zip(mb, numels)] for mb in grads]
         host_outs = [torch.empty_like(p) for p in host_params]
         host_accs = [[torch.zeros(n // W, dtype=torch.float32) for _ in range(W)] for n in numels]
         host_shards = [list(p.view(W, -1)) for p in host_params]
@@ -339,6 +349,9 @@ def main():
     def mean_ms(label):
         return statistics.fmean(durations[label]) if durations[label] else None
 
+    def measured_traffic(kernel):
+        return MEASURED_TRAFFIC_BYTES.get((kernel, args.layout, W)) if args.workload == "layer" else None
+
     g_ms, a_ms, c_ms, s_ms = mean_ms("gather"), mean_ms("accum"), mean_ms("clear"), mean_ms("store")
     if os.environ.get("ODC_BENCH_DEBUG"):
         print("gather ms per launch:", [round(x, 3) for x in durations["gather"]], file=sys.stderr)
@@ -350,6 +363,10 @@ def main():
     value = args.steps * step_bytes / elapsed / 1e9
     workload = (f"cfg2: Llama-3-8B decoder layer ({N} bf16 params, {len(keys)} tensors, "
                 f"{args.layout}), W={W} virtual shards, {MICROBATCHES} microbatches per minibatch")
+    if args.workload == "uneven":
+        workload = (f"cfg3: {len(keys)} flat bf16 parameters of log-uniform size ({sum(valid)} elements, "
+                    f"{N} with the zero padding of the shards), none divisible by W={W}, "
+                    f"{MICROBATCHES} microbatches per minibatch")
     result = {
         "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for gather + scatter-accum, 8B layer, W=8",
         "value": round(value, 1),
@@ -374,7 +391,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(accum_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(("accum", args.layout, W)),
+            "traffic": measured_traffic("accum"),
             "algorithmic_bytes": 10 * N,
             "avg_launch_ms": round(a_ms, 5),
             "min_launch_ms": round(min(durations["accum"]), 5),
@@ -387,7 +404,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gather_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(("gather", args.layout, W)),
+            "traffic": measured_traffic("gather"),
             "algorithmic_bytes": 4 * N,
             "avg_launch_ms": round(g_ms, 5),
             "min_launch_ms": round(min(durations["gather"]), 5),
@@ -397,7 +414,7 @@ def main():
                   "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},
         "store": {"avg_launch_ms": round(s_ms, 5) if s_ms else None,
                   "GB/s": round(6 * N / (s_ms * 1e-3) / 1e9, 1) if s_ms else None,
-                  "traffic": MEASURED_TRAFFIC_BYTES.get(("store", args.layout, W)) if s_ms else None},
+                  "traffic": measured_traffic("store") if s_ms else None},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 4),
         "other_clear_mode": other,
         "cpu_baseline": cpu_baseline,
