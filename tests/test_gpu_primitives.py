@@ -347,3 +347,49 @@ def test_services_called_from_several_host_threads(make_world):
             oracle.scatter_accumulate(want, grads[t][m])
         for r, acc in enumerate(reduction.get_peer_accumulations(("k", t))):
             assert_bit_equal(acc, want[r], f"thread {t}: accumulation of rank {r}")
+
+
+@pytest.mark.parametrize("policy", ["caller", "dedicated"])
+def test_launch_stream_policies(make_world, monkeypatch, policy):
+    """ODC_COMM_STREAM=caller launches on the caller's current stream, =dedicated hops to the one
+    comm stream with joins on both sides (gather.py:114,176): either way a call is ordered like
+    work on the caller's stream, from the default stream and from a side stream alike, and
+    ``sync`` waits for everything launched."""
+    from odc_amd.primitives import utils
+
+    monkeypatch.setenv("ODC_COMM_STREAM", policy)
+    W, S = 8, 30_011
+    group = make_world(W, 16 << 20)
+    gather, reduction, registry = services()
+    g = torch.Generator().manual_seed(11)
+    shards = [(torch.randn(S, generator=g) * 0.02).bfloat16() for _ in range(W)]
+    src = put_shards(registry, "p", shards, group)
+    grads = [(torch.randn(W * S, generator=g) * 1e-3).bfloat16() for _ in range(4)]
+    want = [torch.zeros(S) for _ in range(W)]
+    side = torch.cuda.Stream()
+    out = torch.empty(W * S, dtype=torch.bfloat16, device="cuda")
+    for m, grad in enumerate(grads):
+        dev = grad.cuda()
+        stream = side if m % 2 else torch.cuda.current_stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            src.add_(0.5)  # producer on the caller's stream right before the call
+            gather.gather_into_tensor(out, src, group)
+            doubled = out.float() * 2  # consumer on the caller's stream right after it
+            reduction.scatter_accumulate("k", dev, group)
+        torch.cuda.current_stream().wait_stream(stream)
+        shards[0] = (shards[0].float() + 0.5).bfloat16()
+        oracle.scatter_accumulate(want, grad)
+        assert_bit_equal(doubled, oracle.gather(shards).float() * 2, f"{policy}: microbatch {m}")
+    launched_on = set(utils._launch_streams)
+    if policy == "dedicated":
+        assert launched_on == {utils.get_comm_stream().cuda_stream}
+    else:
+        assert side.cuda_stream in launched_on
+    reduction.sync(group)
+    assert not utils._launch_streams
+    for r, acc in enumerate(reduction.get_peer_accumulations("k")):
+        assert_bit_equal(acc, want[r], f"{policy}: accumulation of rank {r}")
+    monkeypatch.setenv("ODC_COMM_STREAM", "sideways")
+    with pytest.raises(ValueError):
+        gather.gather_into_tensor(out, src, group)
