@@ -72,7 +72,7 @@ class GatherService:
                 items[i].shard_bytes = inp.numel() * inp.element_size()
 
         lib = _native.load()
-        with comm_stream_section() as comm:
+        with comm_stream_section(f"odc.gather[{len(items)}]") as comm:
             stream = ctypes.c_void_p(comm.cuda_stream)
             if cast:
                 # shards kept in one dtype (fp32 master copies), full parameter wanted in another

@@ -87,7 +87,7 @@ class ReductionService:
             offset, shape, dtype = registry.offsets[self._acc_key(key)]
             spans[i].offset = offset
             spans[i].nbytes = shape[0] * dtype.itemsize
-        with comm_stream_section() as comm:
+        with comm_stream_section("odc.clear") as comm:
             _native.check(
                 _native.load().odc_clear(
                     get_world().arena.handle, spans, len(spans), ctypes.c_void_p(comm.cuda_stream)
@@ -116,7 +116,7 @@ class ReductionService:
             return
         lib = _native.load()
         entry = lib.odc_scatter_store if store else lib.odc_scatter_accumulate
-        with comm_stream_section() as comm:
+        with comm_stream_section("odc.scatter_store" if store else "odc.scatter_accumulate") as comm:
             _native.check(
                 entry(
                     get_world().arena.handle,
@@ -300,7 +300,7 @@ class ReductionService:
                 items[i].out = out.data_ptr()
                 results.append(out)
         target = acc_dtype if out_dtype is None else out_dtype
-        with comm_stream_section() as comm:
+        with comm_stream_section("odc.publish") as comm:
             _native.check(
                 _native.load().odc_publish(
                     get_world().arena.handle,

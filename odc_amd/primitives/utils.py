@@ -489,9 +489,16 @@ def launch_stream_policy() -> str:
     return policy
 
 
+def _tracing() -> bool:
+    return os.environ.get("ODC_TRACE", "0") == "1"
+
+
 @contextlib.contextmanager
-def comm_stream_section():
-    """The stream the body's launches go to.
+def comm_stream_section(label: str = "odc"):
+    """The stream the body's launches go to. With ``ODC_TRACE=1`` the section is a marker
+    range named ``label`` (roctx through ``torch.cuda.nvtx``; the reference brackets the same
+    places with NVTX, ``scatter_accumulate.py:307,383,736``), visible to
+    ``rocprofv3 --marker-trace``.
 
     The reference hops to its comm stream and joins it with the current stream on both sides
     (``gather.py:114,176``; ``scatter_accumulate.py:636-640,725-727``), which orders a launch
@@ -500,21 +507,28 @@ def comm_stream_section():
     streams, and on this GPU every extra hardware queue with event joins in flight slows the
     dispatch of all queues (measured on a Llama layer stack: 28.8 -> 22.4 ms per microbatch).
     ``ODC_COMM_STREAM=dedicated`` restores the hop."""
-    current = torch.cuda.current_stream()
-    if launch_stream_policy() == "caller":
-        _launch_streams[current.cuda_stream] = current
-        yield current
-        return
-    comm = get_comm_stream()
-    _launch_streams[comm.cuda_stream] = comm
-    if current == comm:
-        yield comm
-        return
-    comm.wait_stream(current)
+    traced = _tracing()
+    if traced:
+        torch.cuda.nvtx.range_push(label)
     try:
-        yield comm
+        current = torch.cuda.current_stream()
+        if launch_stream_policy() == "caller":
+            _launch_streams[current.cuda_stream] = current
+            yield current
+            return
+        comm = get_comm_stream()
+        _launch_streams[comm.cuda_stream] = comm
+        if current == comm:
+            yield comm
+            return
+        comm.wait_stream(current)
+        try:
+            yield comm
+        finally:
+            current.wait_stream(comm)
     finally:
-        current.wait_stream(comm)
+        if traced:
+            torch.cuda.nvtx.range_pop()
 
 
 def wait_for_launches() -> None:
