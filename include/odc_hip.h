@@ -205,7 +205,7 @@ const char* odc_last_error(void);
 int odc_abi_version(void);
 
 /* Launch-shape knobs, for measurement. "gather_blocks_per_cu", "accum_blocks_per_cu",
- * "store_blocks_per_cu", "clear_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
+ * "store_blocks_per_cu", "clear_blocks_per_cu", "publish_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
  * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
  * "cast_resident_cap", "accum_resident_cap", "store_resident_cap": for one-workgroup-per-tile
  * launches, the most workgroups resident per CU

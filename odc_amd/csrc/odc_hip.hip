@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -74,6 +75,7 @@ struct Options {
   int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
   int64_t store_resident_cap = 4;
   int64_t clear_blocks_per_cu = 0;
+  int64_t publish_blocks_per_cu = 0;
   int64_t rank_major = 1;
   int64_t rank_stagger_bytes = 0;
 };
@@ -85,6 +87,7 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "gather_blocks_per_cu")) return &g_opt.gather_blocks_per_cu;
   if (!strcmp(name, "accum_blocks_per_cu")) return &g_opt.accum_blocks_per_cu;
   if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
+  if (!strcmp(name, "publish_blocks_per_cu")) return &g_opt.publish_blocks_per_cu;
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
   if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
   if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
@@ -167,7 +170,8 @@ struct PublishLaunch {  // one rank's region only: tt.world == 1
   TileTable tt;
   uint8_t* region;      // base of the publishing rank's region
   float divisor;
-  uint32_t divide;      // 0: leave the accumulation untouched
+  float reciprocal;     // exact 1 / divisor when divide == 2
+  uint32_t divide;      // 0: leave the accumulation untouched, 1: divide, 2: multiply by reciprocal
   uint8_t* out[kMaxItems];  // may be null: divide in place only
   uint64_t acc_off[kMaxItems];
   uint64_t seg_elems[kMaxItems];
@@ -631,8 +635,13 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
         float f[4];
         Quad<A>::widen(raw[u], f);
         if (launch.divide) {
+          if (launch.divide == 2) {
 #pragma unroll
-          for (int k = 0; k < 4; ++k) f[k] = f[k] / launch.divisor;
+            for (int k = 0; k < 4; ++k) f[k] = f[k] * launch.reciprocal;
+          } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) f[k] = f[k] / launch.divisor;
+          }
           raw[u] = Quad<A>::narrow(f);
           __builtin_nontemporal_store(raw[u], ap + u * kThreads);
           Quad<A>::widen(raw[u], f);  // the copy is a cast of the ROUNDED accumulation
@@ -652,7 +661,8 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
         const uint32_t i = j * kThreads + tid;
         if (i < n) {
           if (launch.divide) {
-            raw[j] = Codec<A>::narrow(Codec<A>::widen(raw[j]) / launch.divisor);
+            const float x = Codec<A>::widen(raw[j]);
+            raw[j] = Codec<A>::narrow(launch.divide == 2 ? x * launch.reciprocal : x / launch.divisor);
             acc[i] = raw[j];
           }
           if (out) out[i] = Codec<O>::narrow(Codec<A>::widen(raw[j]));
@@ -1297,6 +1307,15 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
     L.region = region;
     L.divisor = divisor;
     L.divide = divisor != 1.0f;
+    L.reciprocal = 1.0f;
+    // Dividing by a power of two whose reciprocal is a normal number is the same correctly
+    // rounded result as multiplying by that reciprocal (both round one exact real value), and
+    // costs one instruction instead of the division sequence.
+    int exponent = 0;
+    if (L.divide && std::fabs(std::frexp(divisor, &exponent)) == 0.5f && exponent > -120 && exponent < 120) {
+      L.reciprocal = 1.0f / divisor;
+      L.divide = 2;
+    }
     L.tt.rank_major = 1u;
     L.tt.first_rank = 0;
     const int n = fill_tile_table(
@@ -1308,7 +1327,8 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
         });
     if (n < 0) return n;
     if (n == 0) continue;
-    const uint32_t grid = grid_for(a, opt.accum_blocks_per_cu, L.tt.n_tiles);
+    // one workgroup per tile: the division sequence wants the occupancy, and the launch is short
+    const uint32_t grid = grid_for(a, opt.publish_blocks_per_cu, L.tt.n_tiles);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }

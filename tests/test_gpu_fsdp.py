@@ -126,3 +126,16 @@ def test_fsdp2_group_layout(make_world, W, fused, dtype):
     del got, unsharded, pgp
     fsdp2.stop()  # fsdp2.py:1141-1144
     assert not utils.is_initialized()
+
+
+def test_group_paths_example_runs():
+    """examples/fsdp2_group_paths.py (reference data flow against the fused one, timed) runs to
+    the end; equality of the two flows is what test_fsdp2_group_layout checks."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    script = Path(__file__).resolve().parent.parent / "examples" / "fsdp2_group_paths.py"
+    proc = subprocess.run([sys.executable, str(script), "--iters", "3"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    assert "publish" in proc.stdout and "unshard" in proc.stdout
