@@ -182,3 +182,47 @@ def test_config5_full_llama3_8b_sweep(make_world):
                 oracle.scatter_accumulate(accs, g1.cpu())
                 assert_bit_equal(got, torch.cat(accs), f"unit {u} param {p} vs oracle")
             del g0, g1, expect, got
+
+
+@pytest.mark.parametrize("W", [8, 12])
+def test_layer_with_fp32_master_shards_cast_gather_and_publish(make_world, W):
+    """The layer at full size the way FSDP mixed precision runs it: fp32 master shards gathered
+    as bf16 in one pass (against torch's own CPU ``.to(bfloat16)`` of the concatenation), bf16
+    gradients into fp32 accumulations, then the end-of-minibatch divide by W and bf16 copy
+    (against the oracle's torch CPU division and cast). W=12 divides with a true division."""
+    from odc_amd import virtual_rank
+
+    shapes = llama3_8b_layer_shapes()
+    numels = [numel(s) for _, s in shapes]
+    S = [shard_numel(n, W) for n in numels]
+    group = make_world(W, sum(s * 8 + 512 for s in S) + (1 << 20))
+    gather, reduction, registry = _services()
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    keys = list(range(len(numels)))
+    shards = []
+    for key, s in zip(keys, S):
+        registry.allocate_symm_buffer(key, (s,), torch.float32)
+        for peer in registry.peer_tensors[key]:
+            peer.normal_(0.0, 0.02, generator=gen)
+        shards.append([p.cpu() for p in registry.peer_tensors[key]])
+    outs = [torch.empty(W * s, dtype=torch.bfloat16, device="cuda") for s in S]
+    with virtual_rank(W - 1):
+        gather.gather_into_tensors(outs, [registry.get_symm_buffer(k) for k in keys], group)
+    for o, sh in zip(outs, shards):
+        assert_bit_equal(o, torch.cat(sh).to(torch.bfloat16), "converting gather")
+    del outs
+
+    want = [[torch.zeros(s) for _ in range(W)] for s in S]
+    for _ in range(2):
+        grads = [device_randn_bf16(W * s, gen, 1e-3) for s in S]
+        reduction.scatter_accumulate_multi(keys, grads, group)
+        for accs, g in zip(want, grads):
+            oracle.scatter_accumulate(accs, g.cpu())
+    reduction.sync(group)
+    for rank in (0, W - 1):
+        with virtual_rank(rank):
+            published = reduction.publish(keys, out_dtype=torch.bfloat16, divisor=float(W))
+            for key, out, accs in zip(keys, published, want):
+                averaged = oracle.fsdp2_average(accs[rank].clone(), W)
+                assert_bit_equal(reduction.get_accumulation(key), averaged, f"rank {rank} key {key}: acc / W")
+                assert_bit_equal(out, averaged.to(torch.bfloat16), f"rank {rank} key {key}: bf16 copy")
