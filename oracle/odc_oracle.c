@@ -103,3 +103,12 @@ void oracle_widen_f16(float* out, const uint16_t* in, uint64_t n) {
 void oracle_narrow_bf16(uint16_t* out, const float* in, uint64_t n) {
   for (uint64_t i = 0; i < n; ++i) out[i] = narrow_bf16(in[i]);
 }
+
+/* acc[i] /= divisor: one binary32 division, correctly rounded (the divide of
+ * odc/fsdp/fsdp2.py:846-847 and of _div_if_needed, odc/fsdp/fsdp1.py:324-330). */
+void oracle_divide_f32(float* acc, float divisor, uint64_t n) {
+  for (uint64_t i = 0; i < n; ++i) {
+    volatile float q = acc[i] / divisor;
+    acc[i] = q;
+  }
+}

@@ -11,7 +11,10 @@ repository (sail-sg/odc) or, where marked ``torch/``, in the PyTorch the referen
 How each function is pinned (tests/test_oracle.py):
   gather_cast               fp32->bf16 against the C restatement's integer round-to-nearest-even
                             on random values, ties and every exponent; widening casts are exact.
-  fsdp1_publish / fsdp2_average   torch CPU div_ against numpy float32 division.
+  fsdp1_publish / fsdp2_average   torch CPU div_ against exact rational arithmetic (fractions) on
+                            samples and against the C restatement's binary32 division on random
+                            values, denormals, zeros and infinities; the bf16 copy against the C
+                            integer rounding.
   gather_into_tensor        closed-form ``i + 2r`` pattern of examples/all_gather.py:80-84,121-125;
                             brute-force Python loops on tiny inputs; sentinel bytes around dst.
   scatter_accumulate        closed forms (ones x M == M, powers of two, +0 + -0 == +0, Inf/NaN);

@@ -30,6 +30,7 @@ def c_oracle():
     lib.oracle_widen_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
     lib.oracle_widen_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
     lib.oracle_narrow_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
+    lib.oracle_divide_f32.argtypes = [ctypes.c_void_p, ctypes.c_float, ctypes.c_uint64]
     return lib
 
 
@@ -342,3 +343,68 @@ def test_publish_rules():
     assert torch.equal(oracle.fsdp1_publish(acc.clone(), 8.0, torch.bfloat16), torch.tensor([1.0, -0.5, 0.125]).bfloat16())
     assert torch.equal(oracle.fsdp1_publish(acc.clone(), 1.0, torch.float32), acc)  # factor <= 1: no divide
     assert torch.equal(oracle.fsdp2_average(acc.clone(), 4), acc / 4)
+
+
+def _nearest_f32(exact):
+    """Round an exact Fraction to binary32, nearest even, by looking at the neighbours of the
+    float64-rounded guess (no floating-point arithmetic decides the result)."""
+    import numpy as np
+    from fractions import Fraction
+
+    guess = np.float32(float(exact))
+    candidates = {guess, np.nextafter(guess, np.float32(-np.inf)), np.nextafter(guess, np.float32(np.inf))}
+    best = None
+    for c in candidates:
+        if not np.isfinite(c):
+            continue
+        err = abs(Fraction(float(c)) - exact)
+        even = (int(np.array(c, dtype=np.float32).view(np.uint32)) & 1) == 0
+        key = (err, 0 if even else 1)
+        if best is None or key < best[0]:
+            best = (key, c)
+    return best[1]
+
+
+@pytest.mark.parametrize("divisor", [3.0, 8.0, 12.0, 64.0, 7.0])
+def test_publish_division_is_correctly_rounded(divisor, c_oracle):
+    """The oracle's divide (torch CPU ``/=``) against exact rational arithmetic on samples and
+    against the C restatement on a large random set incl. denormals, zeros, infinities: the end
+    of minibatch divide has ONE answer per element, which the HIP kernel must reproduce (a
+    multiply by a rounded reciprocal differs for divisors that are not powers of two)."""
+    import numpy as np
+    from fractions import Fraction
+
+    g = torch.Generator().manual_seed(int(divisor))
+    x = torch.cat([
+        torch.randn(200_000, generator=g) * 1e-3,
+        torch.randn(1000, generator=g) * 1e-40,  # results in the denormal range
+        torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1.0, 3.0, 1e-45, 3.4e38]),
+        torch.arange(1, 2000, dtype=torch.float32),
+    ])
+    got = oracle.fsdp2_average(x.clone(), divisor)
+    via_c = x.clone()
+    c_oracle.oracle_divide_f32(via_c.data_ptr(), divisor, via_c.numel())
+    assert torch.equal(_bits(got), _bits(via_c))
+    assert torch.equal(_bits(oracle.fsdp1_publish(x.clone(), divisor, torch.float32)), _bits(via_c))
+    for i in list(range(0, 200_000, 997)) + list(range(200_000, 201_000, 13)) + list(range(201_008, x.numel(), 41)):
+        xi = float(x[i])
+        want = _nearest_f32(Fraction(xi) / Fraction(divisor))
+        assert np.float32(got[i].item()).view(np.uint32) == np.float32(want).view(np.uint32), (i, xi)
+    if divisor not in (8.0, 64.0):  # the shortcut that is NOT allowed: multiply by the rounded reciprocal
+        shortcut = x * torch.tensor(1.0 / divisor, dtype=torch.float32)
+        finite = torch.isfinite(x)
+        assert not torch.equal(_bits(shortcut[finite]), _bits(got[finite]))
+    else:  # for powers of two the reciprocal is exact and the product is the same rounding
+        assert torch.equal(_bits(x * (1.0 / divisor)), _bits(got))
+
+
+def test_bf16_copy_of_the_accumulation_rounds_to_nearest_even(c_oracle):
+    """``acc.to(bfloat16)`` (odc/fsdp/fsdp1.py:331-335, fsdp2.py:897-899) against the integer
+    rounding of the C restatement, ties and the overflow to infinity included."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.cat([torch.randn(100_000, generator=g), torch.randn(1000, generator=g) * 1e-39,
+                   torch.tensor([1.00390625, 1.01171875, 3.3895314e38, 3.4e38, -3.4e38, 0.0, -0.0])])
+    out = torch.empty(x.numel(), dtype=torch.int16)
+    c_oracle.oracle_narrow_bf16(out.data_ptr(), x.data_ptr(), x.numel())
+    assert torch.equal(out, _bits(x.to(torch.bfloat16)))
+    assert torch.isinf(x.to(torch.bfloat16)[-4:-2]).all()  # 3.4e38 rounds up to infinity
