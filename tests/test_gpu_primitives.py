@@ -73,7 +73,7 @@ def test_config1_plumbing(make_world):
         assert_bit_equal(acc, torch.zeros(N // W), "cleared accumulation")
 
 
-@pytest.mark.parametrize("W", [1, 2, 3, 5, 8, 12, 64])
+@pytest.mark.parametrize("W", [1, 2, 3, 5, 8, 12, 64, 200])
 @pytest.mark.parametrize("S", [0, 1, 7, 63, 64, 65, 4095, 4096, 4097, 16384 + 3, 100_003])
 def test_gather_any_shard_size(make_world, W, S):
     """Byte copy at every alignment: odd shard sizes put block r of the output at odd offsets."""
@@ -101,7 +101,7 @@ def test_gather_any_shard_size(make_world, W, S):
     (torch.bfloat16, torch.bfloat16),
     (torch.float16, torch.float16),
 ])
-@pytest.mark.parametrize("W,S", [(1, 5), (4, 1), (8, 4096), (8, 4099), (12, 33_337), (3, 70_001)])
+@pytest.mark.parametrize("W,S", [(1, 5), (4, 1), (8, 4096), (8, 4099), (12, 33_337), (3, 70_001), (200, 4_101)])
 def test_scatter_accumulate_dtypes_and_sizes(make_world, grad_dtype, acc_dtype, W, S):
     from odc_amd import ReductionService
 
