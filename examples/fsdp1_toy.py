@@ -37,9 +37,10 @@ def main():
     ap.add_argument("--layers", type=int, default=2)
     ap.add_argument("--forward-prefetch", action="store_true")
     ap.add_argument("--no-backward-prefetch", action="store_true")
+    ap.add_argument("--shard-grad-op", action="store_true", help="ZeRO-2: keep parameters unsharded between forward and backward")
     args = ap.parse_args()
 
-    from torch.distributed.fsdp import BackwardPrefetch, MixedPrecision
+    from torch.distributed.fsdp import BackwardPrefetch, MixedPrecision, ShardingStrategy
     from torch.distributed.fsdp import FullyShardedDataParallel as FSDP
     from torch.distributed.fsdp._common_utils import clean_tensor_name
     from torch.distributed.fsdp.wrap import ModuleWrapPolicy
@@ -65,6 +66,7 @@ def main():
         device_id=torch.cuda.current_device(),
         use_orig_params=False,
         forward_prefetch=args.forward_prefetch,
+        sharding_strategy=ShardingStrategy.SHARD_GRAD_OP if args.shard_grad_op else ShardingStrategy.FULL_SHARD,
         backward_prefetch=None if args.no_backward_prefetch else BackwardPrefetch.BACKWARD_PRE,
     )
     units = []  # (flat-parameter handle, names of the original parameters in flat order)

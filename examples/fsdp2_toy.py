@@ -78,6 +78,8 @@ def main():
     ap.add_argument("--world-size", type=int, default=8)
     ap.add_argument("--mixed-precision", action="store_true")
     ap.add_argument("--explicit-prefetching", action="store_true")
+    ap.add_argument("--no-reshard-after-forward", action="store_true",
+                    help="ZeRO-2: keep parameters unsharded between forward and backward")
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--microbatches", type=int, default=2)
     ap.add_argument("--layers", type=int, default=2)
@@ -103,7 +105,7 @@ def main():
     unsharded = copy.deepcopy(model)
     full_params = {n: p.detach().clone() for n, p in unsharded.named_parameters()}
 
-    kwargs = {"mesh": mesh}
+    kwargs = {"mesh": mesh, "reshard_after_forward": not args.no_reshard_after_forward}
     compute_dtype = torch.float32
     if args.mixed_precision:
         kwargs["mp_policy"] = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
