@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--microbatches", type=int, default=2)
     ap.add_argument("--layers", type=int, default=2)
+    ap.add_argument("--sync-every", type=int, default=1,
+                    help="reduce gradients only every so many microbatches (set_requires_gradient_sync); in "
+                         "between they add up unsharded, in the compute dtype")
     args = ap.parse_args()
 
     from torch.distributed.device_mesh import init_device_mesh
@@ -140,14 +143,20 @@ def main():
         if args.explicit_prefetching:
             model.unshard()
         want = {n: torch.zeros_like(full_params[n], dtype=torch.float32) for n in names}
-        for _ in range(args.microbatches):
+        pending = {}  # gradients not reduced yet: FSDP keeps their sum unsharded, in the reduce dtype (fp32)
+        for m in range(args.microbatches):
+            sync = (m + 1) % args.sync_every == 0 or m + 1 == args.microbatches
+            model.set_requires_gradient_sync(sync)
             tokens = torch.randint(0, vocab, (batch, seq), device="cuda", generator=data)
             loss = F.cross_entropy(model(tokens).float().view(-1, vocab), tokens.view(-1))
             loss.backward()
             twin.zero_grad(set_to_none=True)
             F.cross_entropy(twin(tokens).float().view(-1, vocab), tokens.view(-1)).backward()
             for n, p in twin.named_parameters():
-                want[n].add_(p.grad)  # fp32 += compute-dtype gradient, in microbatch order
+                pending[n] = p.grad.float() if n not in pending else pending[n] + p.grad.float()
+            if sync:
+                for n in names:
+                    want[n].add_(pending.pop(n))  # fp32 += what reaches the reduction, in order
         fsdp2.pre_optimizer_step(model)
         for n, p in model.named_parameters():
             got = p.grad._local_tensor
