@@ -13,6 +13,7 @@ runs beside it; rank 0's flat gradient shards must equal it bit for bit at every
 from __future__ import annotations
 
 import argparse
+import contextlib
 import copy
 import math
 import sys
@@ -37,6 +38,9 @@ def main():
     ap.add_argument("--layers", type=int, default=2)
     ap.add_argument("--forward-prefetch", action="store_true")
     ap.add_argument("--no-backward-prefetch", action="store_true")
+    ap.add_argument("--sync-every", type=int, default=1,
+                    help="reduce gradients only every so many microbatches (no_sync() in between: the "
+                         "unsharded bf16 gradients add up in place)")
     ap.add_argument("--shard-grad-op", action="store_true", help="ZeRO-2: keep parameters unsharded between forward and backward")
     args = ap.parse_args()
 
@@ -95,12 +99,17 @@ def main():
                     off += named[f].numel()
         twin = copy.deepcopy(unsharded).bfloat16()
         want = [None] * len(units)
-        for _ in range(args.microbatches):
+        twin.zero_grad(set_to_none=True)
+        for m in range(args.microbatches):
+            sync = (m + 1) % args.sync_every == 0 or m + 1 == args.microbatches
             tokens = torch.randint(0, vocab, (batch, seq), device="cuda", generator=data)
-            loss = F.cross_entropy(fsdp_model(tokens).float().view(-1, vocab), tokens.view(-1))
-            loss.backward()
-            twin.zero_grad(set_to_none=True)
+            with contextlib.nullcontext() if sync else fsdp_model.no_sync():
+                loss = F.cross_entropy(fsdp_model(tokens).float().view(-1, vocab), tokens.view(-1))
+                loss.backward()
+            # the twin's gradients add up in bf16 between reductions, as the unsharded flat gradient does
             F.cross_entropy(twin(tokens).float().view(-1, vocab), tokens.view(-1)).backward()
+            if not sync:
+                continue
             grads = dict(twin.named_parameters())
             for u, (handle, fqns) in enumerate(units):
                 flat_grad = torch.cat([grads[f].grad.reshape(-1) for f in fqns])
@@ -109,6 +118,7 @@ def main():
                 chunk = math.ceil(flat_grad.numel() / W)
                 mine = flat_grad[:chunk].float()
                 want[u] = (torch.zeros_like(mine) if want[u] is None else want[u]) + mine  # first add is +0 + g
+            twin.zero_grad(set_to_none=True)
         fsdp1.pre_optimizer_step(fsdp_model)
         for u, (handle, fqns) in enumerate(units):
             expect = want[u]

@@ -120,6 +120,7 @@ def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, 
     ["--world-size", "12", "--layers", "3", "--forward-prefetch"],
     ["--world-size", "5", "--layers", "2", "--no-backward-prefetch", "--microbatches", "3"],
     ["--world-size", "12", "--layers", "3", "--shard-grad-op"],
+    ["--world-size", "8", "--layers", "2", "--microbatches", "4", "--sync-every", "2"],
 ])
 def test_transformer_example_trains_bit_exactly(extra):
     """examples/fsdp1_toy.py: a small transformer under FSDP1 with forward / backward prefetching
