@@ -77,6 +77,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--world-size", type=int, default=8)
     ap.add_argument("--mixed-precision", action="store_true")
+    ap.add_argument("--reduce-dtype", choices=["fp32", "bf16", "fp16"], default="fp32",
+                    help="with --mixed-precision: the dtype gradients are reduced and accumulated in "
+                         "(fp16 splits the division by W into a pre- and a post-divide)")
     ap.add_argument("--explicit-prefetching", action="store_true")
     ap.add_argument("--no-reshard-after-forward", action="store_true",
                     help="ZeRO-2: keep parameters unsharded between forward and backward")
@@ -109,10 +112,23 @@ def main():
     full_params = {n: p.detach().clone() for n, p in unsharded.named_parameters()}
 
     kwargs = {"mesh": mesh, "reshard_after_forward": not args.no_reshard_after_forward}
-    compute_dtype = torch.float32
+    compute_dtype = reduce_dtype = torch.float32
     if args.mixed_precision:
-        kwargs["mp_policy"] = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
+        reduce_dtype = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[args.reduce_dtype]
+        kwargs["mp_policy"] = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=reduce_dtype)
         compute_dtype = torch.bfloat16
+    # torch's rule (_fsdp_collectives._get_gradient_divide_factors): fp32 / bf16 reduce with AVG, i.e.
+    # one division by W at the end; fp16 divides by ~sqrt(W) before and by the rest after
+    pre_divide, post_divide = None, float(W)
+    if reduce_dtype == torch.float16:
+        pre_divide = 1
+        while W % pre_divide == 0 and W / pre_divide > pre_divide:
+            pre_divide *= 2
+        post_divide = W / pre_divide
+
+    def add_in(acc, x):
+        """acc (reduce dtype) += x: computed in fp32, rounded to acc's dtype, as torch's add_ does."""
+        return (acc.float() + x.float()).to(acc.dtype)
     for layer in model.layers:
         fully_shard(layer, **kwargs)
     fully_shard(model, **kwargs)
@@ -142,8 +158,8 @@ def main():
         twin = copy.deepcopy(unsharded).to(compute_dtype)
         if args.explicit_prefetching:
             model.unshard()
-        want = {n: torch.zeros_like(full_params[n], dtype=torch.float32) for n in names}
-        pending = {}  # gradients not reduced yet: FSDP keeps their sum unsharded, in the reduce dtype (fp32)
+        want = {n: torch.zeros_like(full_params[n], dtype=reduce_dtype) for n in names}
+        pending = {}  # gradients not reduced yet: FSDP keeps their sum unsharded, in the reduce dtype
         for m in range(args.microbatches):
             sync = (m + 1) % args.sync_every == 0 or m + 1 == args.microbatches
             model.set_requires_gradient_sync(sync)
@@ -153,16 +169,19 @@ def main():
             twin.zero_grad(set_to_none=True)
             F.cross_entropy(twin(tokens).float().view(-1, vocab), tokens.view(-1)).backward()
             for n, p in twin.named_parameters():
-                pending[n] = p.grad.float() if n not in pending else pending[n] + p.grad.float()
+                pending[n] = p.grad.to(reduce_dtype) if n not in pending else add_in(pending[n], p.grad)
             if sync:
                 for n in names:
-                    want[n].add_(pending.pop(n))  # fp32 += what reaches the reduction, in order
+                    g = pending.pop(n)
+                    if pre_divide is not None and pre_divide > 1:
+                        g = g / pre_divide  # a power of two: exact but for fp16 underflow
+                    want[n] = add_in(want[n], g)  # what reaches the reduction, in order
         fsdp2.pre_optimizer_step(model)
         for n, p in model.named_parameters():
             got = p.grad._local_tensor
-            # FSDP averages over the W ranks; divided on the host, where torch's division is the
-            # correctly rounded one for every W
-            expect = (local_rows(want[n], W).cpu() / W).cuda()
+            # the last division on the host, where torch's is the correctly rounded one for every W;
+            # the gradient is handed over in the parameters' own dtype (fp32)
+            expect = (local_rows(want[n], W).cpu() / post_divide).float().cuda()
             if not torch.equal(got.view(torch.int32), expect.view(torch.int32)):
                 worst = (got - expect).abs().max().item()
                 raise SystemExit(f"step {step}: gradient shard of {n} differs from the unsharded model (max |d| {worst:g})")

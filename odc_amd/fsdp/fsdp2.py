@@ -403,6 +403,10 @@ def foreach_reduce(fsdp_params, unsharded_grads, reduce_scatter_group, reduce_sc
         for fp, g in zip(fsdp_params, unsharded_grads):
             i = layout.index[id(fp)]
             g = g.contiguous().view(-1)
+            if predivide_factor is not None and predivide_factor > 1 and g.dtype != reduce_dtype:
+                # fp16 reduction of bf16/fp32 gradients: the reference divides AFTER the cast to
+                # the reduce dtype (fsdp2.py:676-690); keep that order of roundings
+                g = g.to(reduce_dtype)
             _div_if_needed(g, predivide_factor)
             g.record_stream(reduce_scatter_stream)  # read there after the caller drops its list
             grads.append(g)

@@ -147,6 +147,9 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
     ["--world-size", "8", "--layers", "2"],
     ["--world-size", "12", "--layers", "3", "--mixed-precision", "--no-reshard-after-forward"],
     ["--world-size", "12", "--layers", "2", "--mixed-precision", "--microbatches", "4", "--sync-every", "2"],
+    ["--world-size", "12", "--layers", "2", "--mixed-precision", "--reduce-dtype", "fp16", "--microbatches", "4",
+     "--sync-every", "2"],  # pre- and post-divide around fp16 accumulations
+    ["--world-size", "8", "--layers", "2", "--mixed-precision", "--reduce-dtype", "bf16", "--microbatches", "3"],
 ])
 def test_transformer_example_trains_bit_exactly(extra):
     """examples/fsdp2_toy.py (the counterpart of examples/FSDP2/example.py): a small transformer
