@@ -47,29 +47,43 @@ class GatherService:
         pairs). Equivalent to calling ``gather_into_tensor`` pair by pair. When the outputs'
         dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)
-        world = get_world()
-        W = group_size(pg)
-        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+        get_world()  # raises when there is no arena (no GPU, or init_nvshmem not called)
         registry = SymmBufferRegistry.get_instance()
         pairs = [(o, i) for o, i in zip(output_tensors, input_tensors) if i.numel() or o.numel()]
         if not pairs:
             return
-        src_dtype, dst_dtype = pairs[0][1].dtype, pairs[0][0].dtype
+        for _, inp in pairs:
+            assert inp.is_cuda and inp.is_contiguous(), "shards are contiguous GPU tensors"
+            assert inp.dtype == pairs[0][1].dtype, "one launch takes one dtype pair"
+        self._gather(
+            [o for o, _ in pairs],
+            [registry.symmetric_offset_of(i) for _, i in pairs],
+            [i.numel() for _, i in pairs],
+            pairs[0][1].dtype,
+            pg,
+        )
+
+    def _gather(self, outs, src_offsets, shard_numels, src_dtype, pg) -> None:
+        """One launch (per 64 items): ``outs[k].view(W, -1)[r]`` = the ``shard_numels[k]`` elements
+        of ``src_dtype`` at symmetric byte offset ``src_offsets[k]`` of rank r."""
+        world = get_world()
+        W = group_size(pg)
+        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+        dst_dtype = outs[0].dtype
         cast = src_dtype != dst_dtype
-        items = ((_native.GatherCastItem if cast else _native.GatherItem) * len(pairs))()
-        for i, (out, inp) in enumerate(pairs):
-            assert out.is_cuda and inp.is_cuda, "gather runs on the GPU only"
-            assert (inp.dtype, out.dtype) == (src_dtype, dst_dtype), "one launch takes one dtype pair"
-            assert out.is_contiguous() and inp.is_contiguous()
-            assert (
-                out.numel() == W * inp.numel()
-            ), f"output numel {out.numel()} != {W} * shard numel {inp.numel()}"
-            items[i].dst = out.data_ptr()
-            items[i].src_offset = registry.symmetric_offset_of(inp)
+        es = src_dtype.itemsize
+        items = ((_native.GatherCastItem if cast else _native.GatherItem) * len(outs))()
+        for item, out, offset, n in zip(items, outs, src_offsets, shard_numels):
+            assert out.is_cuda, "gather runs on the GPU only"
+            assert out.dtype == dst_dtype, "one launch takes one dtype pair"
+            assert out.is_contiguous()
+            assert out.numel() == W * n, f"output numel {out.numel()} != {W} * shard numel {n}"
+            item.dst = out.data_ptr()
+            item.src_offset = offset
             if cast:
-                items[i].shard_elems = inp.numel()
+                item.shard_elems = n
             else:
-                items[i].shard_bytes = inp.numel() * inp.element_size()
+                item.shard_bytes = n * es
 
         lib = _native.load()
         with comm_stream_section(f"odc.gather[{len(items)}]") as comm:
@@ -79,11 +93,11 @@ class GatherService:
                 # (bf16): converted on the way instead of gathered and then cast
                 # (odc/fsdp/fsdp1.py:199-223, odc/fsdp/fsdp2.py:341-343)
                 status = lib.odc_gather_cast(
-                    world.arena.handle, items, len(pairs), native_dtype(src_dtype),
+                    world.arena.handle, items, len(items), native_dtype(src_dtype),
                     native_dtype(dst_dtype), get_rank(), stream,
                 )
             else:
-                status = lib.odc_gather(world.arena.handle, items, len(pairs), get_rank(), stream)
+                status = lib.odc_gather(world.arena.handle, items, len(items), get_rank(), stream)
             _native.check(status)
 
     def gather_slices(
@@ -105,8 +119,13 @@ class GatherService:
         assert len(output_tensors) == len(slice_offsets) == len(slice_numels)
         assert input_tensor.is_cuda and input_tensor.is_contiguous()
         es = input_tensor.element_size()
-        slices = []
-        for off, n in zip(slice_offsets, slice_numels):
+        base = SymmBufferRegistry.get_instance().symmetric_offset_of(input_tensor)
+        outs, offsets, numels = [], [], []
+        for out, off, n in zip(output_tensors, slice_offsets, slice_numels):
             assert 0 <= off and off + n <= input_tensor.numel(), "slice leaves the buffer"
-            slices.append(input_tensor.view(-1)[off : off + n])
-        self.gather_into_tensors(list(output_tensors), slices, pg)
+            if n or out.numel():
+                outs.append(out)
+                offsets.append(base + off * es)
+                numels.append(n)
+        if outs:
+            self._gather(outs, offsets, numels, input_tensor.dtype, pg)
