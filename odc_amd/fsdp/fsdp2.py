@@ -63,6 +63,47 @@ def get_gather_service():
     return gather_service
 
 
+class _GatherWork:
+    """What ``ODCAllGather`` returns for ``async_op=True``: torch calls ``wait()`` on it before
+    the copy-out. The gather was launched on the caller's stream, so the wait is an event."""
+
+    def __init__(self):
+        self.event = torch.cuda.Event()
+        self.event.record()
+
+    def wait(self, timeout=None):
+        torch.cuda.current_stream().wait_event(self.event)
+        return True
+
+
+def _make_odc_all_gather():
+    from torch.distributed.fsdp._fully_shard._fsdp_collectives import AllGather, DefaultAllocMixin
+
+    class ODCAllGather(DefaultAllocMixin, AllGather):
+        """torch's pluggable all-gather (``FSDPModule.set_custom_all_gather``) over the gather
+        primitive, for group buffers that live in the symmetric arena: the reference's class of
+        the same name (fsdp2.py:76-90). ``patch_fsdp2`` does not need it (its ``foreach_all_gather``
+        gathers straight into the parameters); it serves code that keeps torch's copy-in /
+        copy-out and only swaps the collective, and ``input_tensor`` must then be symmetric."""
+
+        def __call__(self, output_tensor, input_tensor, group, async_op=False):
+            get_gather_service().gather_into_tensor(output_tensor, input_tensor, group)
+            return _GatherWork() if async_op else None
+
+    return ODCAllGather
+
+
+_odc_gather_comm = None
+
+
+def get_odc_gather_comm():
+    """The process-wide ``ODCAllGather`` (fsdp2.py:208-212)."""
+    global _odc_gather_comm
+    if _odc_gather_comm is None:
+        _odc_gather_comm = _make_odc_all_gather()()
+    return _odc_gather_comm
+
+
 def get_fsdp_params_key(ids: Sequence[int]) -> str:
     return "fsdp_params_gather_" + "_".join(str(i) for i in ids)
 

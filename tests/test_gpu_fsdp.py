@@ -7,7 +7,7 @@ import types
 import pytest
 import torch
 
-from helpers import assert_bit_equal
+from helpers import assert_bit_equal, put_shards
 from oracle import odc_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -139,3 +139,33 @@ def test_group_paths_example_runs():
     proc = subprocess.run([sys.executable, str(script), "--iters", "3"], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert "publish" in proc.stdout and "unshard" in proc.stdout
+
+
+def test_odc_all_gather_comm_object(make_world):
+    """``ODCAllGather`` (fsdp2.py:76-90): torch's pluggable all-gather protocol over the gather
+    primitive, synchronous and with the work handle of ``async_op=True``."""
+    from odc_amd import SymmBufferRegistry
+    from odc_amd.fsdp import fsdp2
+    from torch.distributed.fsdp._fully_shard._fsdp_api import AllGather
+
+    W, S = 8, 10_007
+    group = make_world(W, 4 << 20)
+    fsdp2.patch_fsdp2()
+    try:
+        comm = fsdp2.get_odc_gather_comm()
+        assert isinstance(comm, AllGather) and comm is fsdp2.get_odc_gather_comm()
+        g = torch.Generator().manual_seed(2)
+        shards = [torch.randn(S, generator=g) for _ in range(W)]
+        src = put_shards(SymmBufferRegistry.get_instance(), "ag", shards)
+        out = comm.allocate((W * S,), dtype=torch.float32, device=torch.device("cuda"))
+        assert comm(out, src, group) is None
+        assert_bit_equal(out, oracle.gather(shards), "synchronous form")
+        out.zero_()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            work = comm(out, src, group, async_op=True)
+        assert work.wait()
+        assert_bit_equal(out, oracle.gather(shards), "async form after wait()")
+    finally:
+        fsdp2.unpatch_fsdp2()
