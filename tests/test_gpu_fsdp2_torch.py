@@ -219,3 +219,21 @@ def test_frozen_and_unused_parameters_get_no_gradient(make_world, fake_process_g
             expect = oracle.fsdp2_average(want[name][: rows * rest].clone(), W).view(p._local_tensor.shape)
             assert_bit_equal(p.grad._local_tensor, expect, f"minibatch {minibatch}: sharded gradient of {name}")
         model.zero_grad(set_to_none=True)
+
+
+def test_llama_architecture_example_checks_bit_exactly():
+    """examples/llama_fsdp2.py --check: Hugging Face's Llama (GQA, RoPE, SwiGLU, RMSNorm; random
+    weights, nothing downloaded) under fully_shard at W=12, every gradient shard against the
+    unsharded model. Skipped where transformers is not installed."""
+    pytest.importorskip("transformers")
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    script = Path(__file__).resolve().parent.parent / "examples" / "llama_fsdp2.py"
+    proc = subprocess.run(
+        [sys.executable, str(script), "--check", "--hidden", "256", "--intermediate", "768", "--heads", "8",
+         "--kv-heads", "2", "--vocab", "2000", "--layers", "2", "--seq", "64", "--world-size", "12", "--steps", "1"],
+        capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    assert "gradient shards match the unsharded model bit for bit" in proc.stdout
