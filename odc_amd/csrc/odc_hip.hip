@@ -107,6 +107,9 @@ int64_t* option_slot(const char* name) {
 #ifndef ODC_TILE_UNROLL
 #define ODC_TILE_UNROLL 4  // independent 16 B accesses per lane per stream before the stores
 #endif
+#ifndef ODC_BODY_ALIGN
+#define ODC_BODY_ALIGN 128  // bytes: alignment of a segment's vector body on the written side
+#endif
 constexpr int kThreads = ODC_TILE_THREADS;
 constexpr int kUnroll = ODC_TILE_UNROLL;
 constexpr int kMaxItems = ODC_MAX_ITEMS_PER_LAUNCH;
@@ -206,7 +209,7 @@ __device__ __forceinline__ TileCoord locate_tile(const TileTable& tt, uint32_t t
 
 // Tile geometry shared by all streaming kernels. A rank segment of `n` units (bytes, or
 // elements) whose written side starts at address D is cut as
-//     head  : the units before the first 16-byte (vector) boundary of D,
+//     head  : the units before the first 128-byte line boundary of D (at most 127 bytes),
 //     body  : nvec whole vectors, written with aligned 128-bit (64-bit for 16-bit outputs) stores,
 //     tail  : what is left after the last whole vector.
 // Tile c owns body vectors [c*kTileVecs, (c+1)*kTileVecs); tile 0 also does the head, and the
@@ -227,7 +230,7 @@ __device__ __forceinline__ V load_stream(const uint8_t* p) {  // nontemporal, an
 }
 
 struct SegShape {
-  uint32_t head;   // units before the first vector boundary (clipped to the segment)
+  uint32_t head;   // units before the first line boundary of the written side (clipped to the segment)
   uint32_t tail;   // units after the last whole vector
   uint64_t nvec;   // whole vectors
   uint64_t last;   // tile that owns the tail
@@ -236,9 +239,13 @@ struct SegShape {
 // unit_bytes: size of one unit; vec_units: units per vector (vec_units * unit_bytes is 8 or 16)
 __device__ __forceinline__ SegShape seg_shape(uintptr_t written_addr, uint64_t n, uint32_t unit_bytes,
                                               uint32_t vec_units) {
-  const uint32_t vec_bytes = unit_bytes * vec_units;
+  // The body starts on a 128 B line of the written side, not merely on a vector boundary: a
+  // wavefront's 64 vector stores then cover whole lines, none shared with the next wavefront.
+  // (The head is at most 127 bytes, i.e. fewer units than a workgroup has lanes.)
+  constexpr uint32_t kLine = ODC_BODY_ALIGN;
+  static_assert(kLine >= 16 && kLine - 1 <= kThreads, "one lane per head unit");
   SegShape g;
-  uint64_t head = ((vec_bytes - (uint32_t)(written_addr & (vec_bytes - 1))) & (vec_bytes - 1)) / unit_bytes;
+  uint64_t head = ((kLine - (uint32_t)(written_addr & (kLine - 1))) & (kLine - 1)) / unit_bytes;
   if (head > n) head = n;
   g.head = (uint32_t)head;
   g.nvec = (n - head) / vec_units;
