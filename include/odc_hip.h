@@ -209,8 +209,10 @@ int odc_abi_version(void);
  * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
  * "cast_resident_cap", "accum_resident_cap", "store_resident_cap": for one-workgroup-per-tile
  * launches, the most workgroups resident per CU
- * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather and scatter-accumulate:
- * 1 = walk a rank's whole shard before the next rank, 0 = interleave ranks tile by tile);
+ * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather; "accum_tile_order" for
+ * scatter-accumulate and scatter-store: 1 = walk a rank's whole shard before the next rank, item by
+ * item, 0 = interleave ranks tile by tile, 2 = rank outermost: all items' segments of rank 0, then of
+ * rank 1, ...; accum_tile_order 3, its default, picks 2 for short segments and 1 otherwise);
  * "rank_stagger_bytes" (extra distance between rank regions, read when an arena is created).
  * Unknown names return ODC_ERR_INVALID. Results never depend on these. */
 int odc_set_option(const char* name, int64_t value);

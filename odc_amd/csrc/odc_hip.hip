@@ -76,7 +76,8 @@ struct Options {
   int64_t store_resident_cap = 4;
   int64_t clear_blocks_per_cu = 0;
   int64_t publish_blocks_per_cu = 0;
-  int64_t rank_major = 1;
+  int64_t rank_major = 1;        // gather: 0 = ranks interleaved, 1 = item-major, 2 = rank outermost
+  int64_t accum_tile_order = 3;  // the same for scatter-accumulate / store; 3 = by segment length
   int64_t rank_stagger_bytes = 0;
 };
 Options g_opt;
@@ -89,6 +90,7 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
   if (!strcmp(name, "publish_blocks_per_cu")) return &g_opt.publish_blocks_per_cu;
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
+  if (!strcmp(name, "accum_tile_order")) return &g_opt.accum_tile_order;
   if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
   if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
   if (!strcmp(name, "cast_resident_cap")) return &g_opt.cast_resident_cap;
@@ -186,21 +188,37 @@ struct TileCoord {
 };
 
 __device__ __forceinline__ TileCoord locate_tile(const TileTable& tt, uint32_t t) {
-  uint32_t lo = 0, hi = tt.n_items;  // largest i with tile_prefix[i] <= t
-  while (hi - lo > 1) {
-    const uint32_t mid = (lo + hi) >> 1;
-    if (tt.tile_prefix[mid] <= t) lo = mid; else hi = mid;
-  }
-  const uint32_t lt = t - tt.tile_prefix[lo];
-  const uint32_t tps = tt.tiles_per_seg[lo];
   TileCoord c;
-  c.item = lo;
-  if (tt.rank_major) {
-    c.rank = lt / tps;
-    c.chunk = lt - c.rank * tps;
+  if (tt.rank_major == 2) {
+    // rank outermost: rank r's segments of all items, then rank r+1's. The arena side of the
+    // launch then walks one rank region from item to item. tile_prefix[i] is world times the
+    // tiles before item i within one rank, so the search compares against lt * world.
+    const uint32_t per_rank = tt.n_tiles / tt.world;
+    c.rank = t / per_rank;
+    const uint64_t lt = (uint64_t)(t - c.rank * per_rank) * tt.world;
+    uint32_t lo = 0, hi = tt.n_items;
+    while (hi - lo > 1) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (tt.tile_prefix[mid] <= lt) lo = mid; else hi = mid;
+    }
+    c.item = lo;
+    c.chunk = (uint32_t)((lt - tt.tile_prefix[lo]) / tt.world);
   } else {
-    c.chunk = lt / tt.world;
-    c.rank = lt - c.chunk * tt.world;
+    uint32_t lo = 0, hi = tt.n_items;  // largest i with tile_prefix[i] <= t
+    while (hi - lo > 1) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (tt.tile_prefix[mid] <= t) lo = mid; else hi = mid;
+    }
+    const uint32_t lt = t - tt.tile_prefix[lo];
+    const uint32_t tps = tt.tiles_per_seg[lo];
+    c.item = lo;
+    if (tt.rank_major) {
+      c.rank = lt / tps;
+      c.chunk = lt - c.rank * tps;
+    } else {
+      c.chunk = lt / tt.world;
+      c.rank = lt - c.chunk * tt.world;
+    }
   }
   c.rank += tt.first_rank;
   if (c.rank >= tt.world) c.rank -= tt.world;
@@ -1093,7 +1111,7 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
     GatherLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.rank_major = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
     const int n = fill_tile_table(
         L.tt, a->world, n_items, &next, kTileBytes, [&](uint32_t i) { return items[i].shard_bytes; },
@@ -1144,7 +1162,7 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     CastGatherLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.rank_major = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
     const int n = fill_tile_table(
         L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
@@ -1234,7 +1252,7 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     AccumLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = opt.rank_major ? 1u : 0u;
+    L.tt.rank_major = (uint32_t)opt.rank_major;
     L.tt.first_rank = 0;
     const int n = fill_tile_table(
         L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
@@ -1246,6 +1264,16 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
         });
     if (n < 0) return n;
     if (n == 0) continue;
+    // Tile order. Item-major (a rank's segment, then the next rank's, item by item) walks the
+    // gradient contiguously and hops between rank regions at every segment; rank-outermost walks
+    // one rank region from accumulation to accumulation (they are neighbours when registered
+    // together) and hops in the gradient instead. The read-modify-write stream is the one worth
+    // keeping contiguous once segments get short (measured: +2.3 % at W=64, +5.7 % on 40 uneven
+    // parameters at W=12, -0.8 % on the layer at W=8, whose segments average 740 tiles).
+    if (opt.accum_tile_order == 3)
+      L.tt.rank_major = (uint64_t)L.tt.n_tiles < 512ull * L.tt.n_items * a->world ? 2u : 1u;
+    else
+      L.tt.rank_major = (uint32_t)opt.accum_tile_order;
     // The persistent shape (one workgroup per CU) streams fastest, but only while every rank's
     // chunk of the gradient and of the accumulation starts on a 128 B line: with nothing else
     // resident to cover for it, a workgroup whose wavefronts straddle lines, or that meets heads,
