@@ -100,3 +100,76 @@ def test_scatter_accumulate_random_slices_and_padding(make_world, seed):
     red.sync(group)
     for r, acc in enumerate(red.get_peer_accumulations("k")):
         assert_bit_equal(acc, want[r], f"seed {seed}: W={W} {grad_dtype}->{acc_dtype} rank {r} sizes {sizes} valid {valid}")
+
+
+KNOBS = [
+    {},
+    {"rank_major": 0, "accum_tile_order": 0},
+    {"rank_major": 2, "accum_tile_order": 2},
+    {"accum_tile_order": 1, "accum_blocks_per_cu": 0, "accum_resident_cap": 0},
+    {"gather_blocks_per_cu": 2, "accum_blocks_per_cu": 3, "store_blocks_per_cu": 1, "clear_blocks_per_cu": 2,
+     "publish_blocks_per_cu": 1},
+    {"gather_resident_cap": 1, "cast_resident_cap": 2, "accum_resident_cap": 8, "store_resident_cap": 0},
+]
+
+
+@pytest.mark.parametrize("knobs", KNOBS, ids=lambda k: ",".join(f"{a}={b}" for a, b in k.items()) or "defaults")
+def test_results_do_not_depend_on_launch_knobs(make_world, knobs):
+    """Every launch-shape and tile-order option on a ragged multi-item workload: gather,
+    converting gather, clear, store form, accumulate and publish must give the oracle's bits
+    whatever the knobs say."""
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry, _native
+
+    names = ["gather_blocks_per_cu", "accum_blocks_per_cu", "store_blocks_per_cu", "clear_blocks_per_cu",
+             "publish_blocks_per_cu", "gather_resident_cap", "cast_resident_cap", "accum_resident_cap",
+             "store_resident_cap", "rank_major", "accum_tile_order"]
+    saved = {n: _native.get_option(n) for n in names}
+    try:
+        for name, value in knobs.items():
+            _native.set_option(name, value)
+        W = 5
+        sizes = [1, 70, 4096, 4099, 16_385, 40_001, 3]
+        group = make_world(W, 8 << 20)
+        registry = SymmBufferRegistry.get_instance()
+        gather, red = GatherService(), ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
+        g = torch.Generator().manual_seed(123)
+        shards = [[torch.randn(s, generator=g) for _ in range(W)] for s in sizes]
+        locals_ = []
+        for i, per_rank in enumerate(shards):
+            registry.allocate_symm_buffer(("p", i), (sizes[i],), torch.float32)
+            for peer, host in zip(registry.peer_tensors[("p", i)], per_rank):
+                peer.copy_(host)
+            locals_.append(registry.get_symm_buffer(("p", i)))
+        outs32 = [torch.empty(W * s, device="cuda") for s in sizes]
+        outs16 = [torch.empty(W * s, dtype=torch.bfloat16, device="cuda") for s in sizes]
+        gather.gather_into_tensors(outs32, locals_, group)
+        gather.gather_into_tensors(outs16, locals_, group)
+        for o32, o16, per_rank in zip(outs32, outs16, shards):
+            assert_bit_equal(o32, oracle.gather(per_rank), "gather")
+            assert_bit_equal(o16, oracle.gather(per_rank).to(torch.bfloat16), "converting gather")
+        keys = list(range(len(sizes)))
+        want = [[torch.zeros(s) for _ in range(W)] for s in sizes]
+        for m in range(3):
+            valid = [max(0, W * s - (m * 7) % (W * s + 1)) for s in sizes]
+            grads = [torch.randn(v, generator=g).bfloat16() for v in valid]
+            if m == 0:
+                for k, s in zip(keys, sizes):
+                    red.register(k, (s,), torch.bfloat16, torch.float32, group)
+            red.scatter_accumulate_multi(keys, [x.cuda() for x in grads], group, valid_numels=valid)
+            for accs, x, s in zip(want, grads, sizes):
+                oracle.scatter_accumulate(accs, torch.cat([x, torch.zeros(W * s - x.numel(), dtype=x.dtype)]))
+        published = red.publish(keys, out_dtype=torch.bfloat16, divisor=3.0)
+        for k, out, accs in zip(keys, published, want):
+            averaged = oracle.fsdp2_average(accs[0].clone(), 3.0)
+            assert_bit_equal(red.get_accumulation(k), averaged, f"key {k}: acc / 3")
+            assert_bit_equal(out, averaged.to(torch.bfloat16), f"key {k}: bf16 copy")
+            for r in range(1, W):
+                assert_bit_equal(red.get_peer_accumulations(k)[r], accs[r], f"key {k} rank {r}")
+        red.lazy_clear = False
+        red.clear_accumulations()
+        for k, s in zip(keys, sizes):
+            for acc in red.get_peer_accumulations(k):
+                assert_bit_equal(acc, torch.zeros(s), "clear")
+    finally:
+        for name, value in saved.items():
+            _native.set_option(name, value)
