@@ -325,3 +325,30 @@ def test_workload_shapes():
     sizes = w.uneven_flat_numels()
     assert len(sizes) == 40 and all(4096 <= n <= 58_720_256 + 12 and n % 12 for n in sizes)
     assert sizes == w.uneven_flat_numels()  # deterministic
+
+
+def test_small_helpers(monkeypatch):
+    """Closed forms and environment lookups that nothing else touches: the splitter's rounding
+    (utils.py:229-230), the node-size lookup (utils.py:195-199) and the symmetric-tensor tag
+    (utils.py:118-124)."""
+    s = utils.BufferSplitter()
+    assert [s.round_to_data_size(n) for n in (0, 1, 63, 64, 65, 100, 128)] == [0, 64, 64, 64, 128, 128, 128]
+    if not utils.is_initialized():
+        monkeypatch.delenv("RAY_LOCAL_WORLD_SIZE", raising=False)
+        monkeypatch.setenv("LOCAL_WORLD_SIZE", "8")
+        assert utils.get_local_world_size() == 8
+        monkeypatch.setenv("RAY_LOCAL_WORLD_SIZE", "4")  # Ray's variable wins, as in the reference
+        assert utils.get_local_world_size() == 4
+        with pytest.raises(RuntimeError):
+            utils.get_world_size()
+    t = torch.zeros(3)
+    assert not utils.SymmBufferRegistry.is_nvshmem_tensor(t)
+    utils.SymmBufferRegistry.set_nvshmem_flag(t)
+    assert utils.SymmBufferRegistry.is_nvshmem_tensor(t)
+    monkeypatch.setenv("ODC_COMM_STREAM", "nonsense")
+    with pytest.raises(ValueError):
+        utils.launch_stream_policy()
+    monkeypatch.setenv("ODC_COMM_STREAM", "dedicated")
+    assert utils.launch_stream_policy() == "dedicated"
+    monkeypatch.delenv("ODC_COMM_STREAM")
+    assert utils.launch_stream_policy() == "caller"
