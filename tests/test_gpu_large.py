@@ -62,3 +62,31 @@ def test_scatter_accumulate_past_two_gi_elements(make_world):
     last = red.get_peer_accumulations("big")[W - 1]
     assert torch.equal(bits(last[: S - 5]), bits(torch.zeros(S - 5, device="cuda").add_(grad[(W - 1) * S : n - 5].float())))
     assert torch.equal(bits(last[S - 5 :]), torch.zeros(5, dtype=torch.int32, device="cuda"))
+
+
+def test_far_end_of_a_128_gib_arena(make_world):
+    """Rank regions of 16 GiB each (the reference's launch script reserves 30 GB per rank):
+    buffers parked at the far end of every region, byte offsets past 2^33 and rank strides past
+    2^34, through gather and both forms of scatter-accumulate."""
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry
+    from odc_amd.primitives import utils
+
+    W, per_rank, n = 8, 16 << 30, 1 << 20
+    group = make_world(W, per_rank)
+    arena = utils.get_world().arena
+    arena.alloc(per_rank - (1 << 30))  # everything after this lands in the last GiB of a region
+    registry = SymmBufferRegistry.get_instance()
+    registry.allocate_symm_buffer("far", (n,), torch.float32)
+    assert registry.get_offset("far") >= per_rank - (1 << 30)
+    for r, peer in enumerate(registry.peer_tensors["far"]):
+        peer.fill_(float(r))
+    out = torch.empty(W * n, device="cuda")
+    GatherService().gather_into_tensor(out, registry.get_symm_buffer("far"), group)
+    assert torch.equal(out.view(W, n), torch.arange(W, dtype=torch.float32, device="cuda")[:, None].expand(W, n))
+    red = ReductionService(accumulation_dtype=torch.float32)
+    grad = torch.arange(W * n, device="cuda").remainder(251).bfloat16()
+    red.scatter_accumulate("k", grad, group)
+    red.scatter_accumulate("k", grad, group)
+    red.sync(group)
+    for r, acc in enumerate(red.get_peer_accumulations("k")):
+        assert torch.equal(acc, grad[r * n : (r + 1) * n].float() * 2), f"rank {r}"
