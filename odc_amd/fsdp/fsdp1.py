@@ -234,7 +234,8 @@ def pre_optimizer_step(fsdp_module):
     service = get_reduction_service()
     factor = getattr(fsdp_module, "_gradient_postdivide_factor", 1.0)
     divisor = factor if factor is not None and factor > 1 else 1.0  # `_div_if_needed`
-    handles = list(fsdp_module._all_handles)
+    # a unit that never saw a gradient (frozen, or unused so far) has no accumulation yet
+    handles = [h for h in fsdp_module._all_handles if id(h.flat_param) in service.accumulation_indices]
     by_dtype = {}
     for handle in handles:
         by_dtype.setdefault(handle.flat_param.dtype, []).append(handle)
