@@ -134,3 +134,60 @@ def test_transformer_example_trains_bit_exactly(extra):
                           capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert proc.stdout.count("match the unsharded model bit for bit") == 3
+
+
+def test_fsdp1_with_a_frozen_unit(make_world, fake_process_group):
+    """A wrapped block none of whose parameters require a gradient never reaches the
+    scatter-accumulate: ``pre_optimizer_step`` leaves its gradient ``None`` and publishes the
+    other units exactly."""
+    from torch.distributed.fsdp import FullyShardedDataParallel as FSDP
+    from torch.distributed.fsdp import MixedPrecision
+    from torch.distributed.fsdp._common_utils import clean_tensor_name
+    from torch.distributed.fsdp.wrap import ModuleWrapPolicy
+
+    from odc_amd.fsdp import fsdp1
+
+    W = 4
+    fake_process_group(W)
+    make_world(W, 64 << 20)
+    fsdp1.patch_fsdp1(reduce_dtype=torch.float32)
+    torch.manual_seed(0)
+    model = Toy().cuda()
+    for p in model.layers[1].parameters():
+        p.requires_grad_(False)
+    reference = copy.deepcopy(model).bfloat16()
+    fsdp_model = FSDP(model, auto_wrap_policy=ModuleWrapPolicy({Block}),
+                      mixed_precision=MixedPrecision(param_dtype=torch.bfloat16),
+                      device_id=torch.cuda.current_device(), use_orig_params=False)
+    units = []
+    for name, module in fsdp_model.named_modules():
+        if isinstance(module, FSDP) and module._handle is not None:
+            prefix = clean_tensor_name(name)
+            units.append((module._handle, [f"{prefix}.{f}" if prefix else f for f in module._handle.flat_param._fqns]))
+    pre, post = fsdp_model._gradient_predivide_factor, fsdp_model._gradient_postdivide_factor
+    g = torch.Generator().manual_seed(2)
+    batches = [torch.randn(16, 32, generator=g).cuda() for _ in range(2)]
+    fsdp1.pre_minibatch_start(fsdp_model)
+    want = {}
+    for x in batches:
+        fsdp_model(x).float().pow(2).mean().backward()
+        reference.zero_grad(set_to_none=True)
+        reference(x.bfloat16()).float().pow(2).mean().backward()
+        grads = {n: p.grad for n, p in reference.named_parameters()}
+        for u, (_, fqns) in enumerate(units):
+            if grads[fqns[0]] is None:
+                continue
+            flat_grad = torch.cat([grads[f].detach().cpu().reshape(-1) for f in fqns])
+            if pre > 1:
+                flat_grad.div_(pre)
+            accs = want.setdefault(u, [torch.zeros(math.ceil(flat_grad.numel() / W)) for _ in range(W)])
+            oracle.scatter_accumulate(accs, oracle.fsdp1_pad_grad(flat_grad, W))
+    fsdp1.pre_optimizer_step(fsdp_model)
+    frozen = [u for u, (_, fqns) in enumerate(units) if fqns[0].startswith("layers.1.")]
+    assert len(frozen) == 1 and frozen[0] not in want
+    for u, (handle, fqns) in enumerate(units):
+        if u in frozen:
+            assert handle.flat_param.grad is None
+        else:
+            expect = oracle.fsdp1_publish(want[u][0].clone(), post, torch.float32)
+            assert_bit_equal(handle.flat_param.grad, expect, f"flat gradient of {fqns[0]}...")
