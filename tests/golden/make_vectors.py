@@ -78,6 +78,8 @@ def main():
     v["fsdp1_grad"] = bits(grad)
     v["fsdp1_acc"] = np.stack([bits(a) for a in accs])
     v["fsdp1_published_div4_bf16"] = bits(oracle.fsdp1_publish(accs[1].clone(), 4.0, torch.bfloat16))
+    # a divisor that is not a power of two: the quotient must be the correctly rounded one
+    v["fsdp2_averaged_div12"] = bits(oracle.fsdp2_average(accs[2].clone(), 12))
     # gather with cast fp32 -> bf16
     W, S = 4, 259
     f32 = [bf16_values(S, 50 + r).float() * 1.00390625 for r in range(W)]  # off the bf16 grid: rounding happens

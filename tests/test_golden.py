@@ -57,6 +57,7 @@ def test_oracle_reproduces_the_vectors(vec):
     for r in range(W):
         assert same_bits(accs[r], vec["fsdp1_acc"][r])
     assert same_bits(oracle.fsdp1_publish(accs[1].clone(), 4.0, torch.bfloat16), vec["fsdp1_published_div4_bf16"])
+    assert same_bits(oracle.fsdp2_average(accs[2].clone(), 12), vec["fsdp2_averaged_div12"])
     f32 = [t(s, torch.float32) for s in vec["cast_shards"]]
     assert same_bits(oracle.gather_cast(f32, torch.bfloat16), vec["cast_out"])
 
@@ -105,6 +106,10 @@ def test_hip_path_reproduces_the_vectors(vec, make_world):
         (published,) = service.publish([id(flat)], out_dtype=torch.bfloat16, divisor=4.0)
         service.sync(group)
         assert same_bits(published, vec["fsdp1_published_div4_bf16"])
+    with virtual_rank(2):
+        service.publish([id(flat)], divisor=12.0)  # in place, a true division
+        service.sync(group)
+        assert same_bits(service.get_accumulation(id(flat)), vec["fsdp2_averaged_div12"])
     for r, s in enumerate(vec["cast_shards"]):
         with virtual_rank(r):
             registry.update_symm_buffer("c", t(s, torch.float32).cuda())
