@@ -8,8 +8,15 @@ One step = one microbatch of the path over the whole layer:
 Every 8th step starts a new minibatch and first clears the accumulations (inside the timed
 region; its 4N written bytes are NOT counted in the numerator).
 
-Prints ONE JSON line: whole-step throughput, per-kernel roofline figures from HIP events on the
-launch stream, the CPU oracle timed on the host cores, and the parity verdict.
+Prints ONE JSON line: whole-step throughput (`value`), per-kernel roofline figures from HIP events
+on the launch stream (`roofline` for the scatter-accumulate, `roofline_gather`), the clear, the
+CPU oracle timed on the host cores (`cpu_baseline`), the parity verdict against that oracle, and
+`other_clear_mode`: the same steps with the services' default lazy clears, where no clear kernel
+runs and the first scatter-accumulate of a minibatch stores instead (6N bytes, counted as such).
+
+Other workloads (not the headline): `--workload uneven --world-size 12` (40 uneven, zero-padded
+flat parameters), `--workload model` (the whole 8.03 G-parameter model), `--layout flat`,
+`--world-size 64`.
 """
 
 from __future__ import annotations
