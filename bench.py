@@ -8,11 +8,20 @@ One step = one microbatch of the path over the whole layer:
 Every 8th step starts a new minibatch and first clears the accumulations (inside the timed
 region; its 4N written bytes are NOT counted in the numerator).
 
-Prints ONE JSON line: whole-step throughput (`value`), per-kernel roofline figures from HIP events
-on the launch stream (`roofline` for the scatter-accumulate, `roofline_gather`), the clear, the
-CPU oracle timed on the host cores (`cpu_baseline`), the parity verdict against that oracle, and
-`other_clear_mode`: the same steps with the services' default lazy clears, where no clear kernel
-runs and the first scatter-accumulate of a minibatch stores instead (6N bytes, counted as such).
+The headline (`value`, `ms_per_step`) times EXACTLY --steps steps replayed from HIP graphs: one
+graph per whole minibatch (clear + 8 x (gather + scatter-accumulate)), one more for the steps left
+over; `--no-graph` launches them eagerly instead. After that, a short eager phase records one HIP
+event on the launch stream after every launch: per-kernel durations for `roofline` (the
+scatter-accumulate, the dominant kernel) and `roofline_gather`.
+
+Prints ONE JSON line with, besides the contract's fields: `roofline.practical_ceiling` (what bare
+streaming kernels of libodc_ceiling.so reach on flat arrays of the same sizes in the same run),
+`roofline.traffic` (HBM bytes per launch from the committed rocprofv3 counter runs listed in
+profiles/traffic.json; null when a launch knob is overridden), `host_us_per_call` (host time of one
+call of each service entry point on the 9-parameter layer), the clear, the CPU oracle timed on
+the host cores (`cpu_baseline`), the parity verdict against that oracle, and `other_clear_mode`:
+the same steps launched eagerly with lazy clears, where no clear kernel runs and the first
+scatter-accumulate of a minibatch stores instead (6N bytes, counted as such).
 
 Other workloads (not the headline): `--workload uneven --world-size 12` (40 uneven, zero-padded
 flat parameters), `--workload model` (the whole 8.03 G-parameter model), `--layout flat`,
@@ -22,6 +31,7 @@ flat parameters), `--workload model` (the whole 8.03 G-parameter model), `--layo
 from __future__ import annotations
 
 import argparse
+import ctypes
 import gc
 import json
 import os
@@ -36,14 +46,7 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 MICROBATCHES = 8
-
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE and
-# WRITE_SIZE runs, scaled by a torch copy kernel of known size); None until measured.
-MEASURED_TRAFFIC_BYTES = {
-    ("accum", "per-param", 8): 2_181_147_887,
-    ("gather", "per-param", 8): 872_565_155,
-    ("store", "per-param", 8): 1_308_913_261,
-}
+TRAFFIC_FILE = ROOT / "profiles" / "traffic.json"
 
 
 def parse_args():
@@ -59,18 +62,28 @@ def parse_args():
                          "parameter model swept unit by unit (needs ~85 GB of HBM; no oracle pass)")
     ap.add_argument("--layout", choices=["per-param", "flat"], default="per-param",
                     help="9 per-parameter shards in one multi-tensor launch, or one flat shard")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch the timed steps eagerly instead of replaying HIP graphs")
+    ap.add_argument("--event-steps", type=int, default=16,
+                    help="eager steps with one HIP event per launch, for the per-kernel roofline figures")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the bare streaming kernels")
+    ap.add_argument("--no-host-overhead", action="store_true", help="skip the host-time-per-call measurement")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline sample length")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--lazy-clear", action="store_true",
-                    help="the services' default mode: no clear kernel, the first scatter-accumulate of a "
-                         "minibatch stores instead (6N bytes); the headline keeps eager clears so that "
-                         "every timed scatter-accumulate is the 10N read-modify-write")
+                    help="lazy clears for the headline: no clear kernel, the first scatter-accumulate of a "
+                         "minibatch stores instead (6N bytes); implies --no-graph (the choice between store "
+                         "and read-modify-write is host state). The default keeps the reference's eager "
+                         "clears, so that every timed scatter-accumulate is the 10N read-modify-write")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="libodc_hip launch knob, e.g. accum_blocks_per_cu=4")
-    return ap.parse_args()
+    args = ap.parse_args()
+    if args.lazy_clear:
+        args.no_graph = True
+    return args
 
 
 def model_sweep(args):
@@ -159,6 +172,114 @@ def model_sweep(args):
     odc_amd.finalize_distributed()
 
 
+def load_traffic(args, W):
+    """HBM bytes per launch from the committed rocprofv3 counter runs: kernel -> (bytes, source).
+    Only for the configuration those runs profiled, and only with the library's default knobs."""
+    if args.option or not TRAFFIC_FILE.exists():
+        return {}
+    try:
+        table = json.loads(TRAFFIC_FILE.read_text())
+    except (OSError, ValueError):
+        return {}
+    out = {}
+    for e in table.get("entries", []):
+        if (e.get("workload"), e.get("layout"), e.get("world_size")) == (args.workload, args.layout, W):
+            out[e["kernel"]] = (e["hbm_bytes_per_launch"],
+                                f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {e['profile']} (not measured by this run)")
+    return out
+
+
+def measure_ceiling(torch, comm, N, iters=12):
+    """Bare streaming kernels over flat arrays of the layer's sizes, launched alternately (copy,
+    read-modify-write, read, write: every launch meets cold caches, as the real steps do) with
+    one HIP event after each. Three launch shapes each; the best average is the ceiling."""
+    from odc_amd import _native
+
+    lib = _native.load_ceiling()
+    src = torch.empty(N, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02)
+    dst = torch.empty_like(src)
+    grad = torch.empty(N, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3)
+    acc = torch.zeros(N, dtype=torch.float32, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    stream = ctypes.c_void_p(comm.cuda_stream)
+    moved = ctypes.c_uint64()
+    shapes = {"one workgroup per tile": (0, 0), "one per tile, 4 resident per CU": (0, 40960),
+              "1 persistent workgroup per CU": (1, 0)}
+
+    def launch(kind, wg, lds):
+        if kind == "copy":
+            rc = lib.odc_ceiling_copy(dst.data_ptr(), src.data_ptr(), 2 * N, wg, lds, stream, ctypes.byref(moved))
+        elif kind == "rmw_bf16_f32":
+            rc = lib.odc_ceiling_rmw(acc.data_ptr(), grad.data_ptr(), N, wg, lds, stream, ctypes.byref(moved))
+        elif kind == "read":
+            rc = lib.odc_ceiling_read(acc.data_ptr(), 4 * N, sink.data_ptr(), wg, lds, stream, ctypes.byref(moved))
+        else:
+            rc = lib.odc_ceiling_write(acc.data_ptr(), 4 * N, wg, lds, stream, ctypes.byref(moved))
+        assert rc == 0, f"ceiling kernel {kind} failed to launch"
+        return moved.value
+
+    kinds = ("copy", "rmw_bf16_f32", "read", "write")
+    table = {k: {} for k in kinds}
+    with torch.cuda.stream(comm):
+        for label, (wg, lds) in shapes.items():
+            marks, nbytes = [], {}
+            for it in range(iters + 2):
+                for kind in kinds:
+                    e0 = torch.cuda.Event(enable_timing=True)
+                    e0.record(comm)
+                    nbytes[kind] = launch(kind, wg, lds)
+                    e1 = torch.cuda.Event(enable_timing=True)
+                    e1.record(comm)
+                    if it >= 2:
+                        marks.append((kind, e0, e1))
+            torch.cuda.synchronize()
+            for kind in kinds:
+                ms = statistics.fmean(a.elapsed_time(b) for k, a, b in marks if k == kind)
+                table[kind][label] = round(nbytes[kind] / (ms * 1e-3) / 1e9, 1)
+    best = {k: max(v.values()) for k, v in table.items()}
+    return {"unit": "GB/s", **best, "by_launch_shape": table,
+            "note": "bare kernels of libodc_ceiling.so on flat arrays of the layer's sizes (copy 2 x 2N bytes, "
+                    "rmw 10N, read 4N, write 4N), launched alternately, HIP events per launch"}
+
+
+def measure_host_overhead(torch, odc_amd, comm, group, gather, reduction, registry, outs, shard_locals, keys,
+                          grads, numels, W, calls=100):
+    """Host time of one call, mean over `calls` back-to-back asynchronous calls (the launches
+    queue up; the device is drained afterwards): the multi-tensor entry points on the 9 tensors,
+    and the slice entry points (the FSDP2 group path) on the same layer as one group buffer."""
+    result = {}
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        dt = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return round(dt / calls * 1e6, 2)
+
+    with torch.cuda.stream(comm):
+        n = len(keys)
+        result[f"gather_into_tensors[{n}]"] = timed(lambda: gather.gather_into_tensors(outs, shard_locals, group))
+        result[f"scatter_accumulate_multi[{n}]"] = timed(
+            lambda: reduction.scatter_accumulate_multi(keys, grads, group))
+        shard_numels = [x // W for x in numels]
+        offsets = [0]
+        for s in shard_numels:
+            offsets.append(offsets[-1] + s)
+        total = offsets.pop()
+        group_buffer = registry.allocate_symm_buffer("bench_group_buffer", (total,), torch.bfloat16)
+        result[f"gather_slices[{n}]"] = timed(
+            lambda: gather.gather_slices(outs, group_buffer, offsets, shard_numels, group))
+        result[f"scatter_accumulate_slices[{n}]"] = timed(
+            lambda: reduction.scatter_accumulate_slices("bench_group", grads, offsets, shard_numels, group,
+                                                        accumulation_numel=total))
+    result["note"] = f"host microseconds per call, mean of {calls} asynchronous calls"
+    return result
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -193,7 +314,7 @@ def main():
     padded = numels != valid
     assert padded == (args.workload == "uneven")
     N = sum(numels)
-    per_rank = sum((n // W) * 6 + 512 for n in numels) + (1 << 20)
+    per_rank = sum((n // W) * 12 + 2048 for n in numels) + (1 << 20)  # shards, accumulations, and the same again as one group
     group = odc_amd.init_nvshmem(world_size=W, symmetric_size=per_rank)
     registry = odc_amd.SymmBufferRegistry.get_instance()
     gather = odc_amd.GatherService()
@@ -211,7 +332,7 @@ def main():
     for key, p in zip(keys, params):
         for r in range(W):
             with odc_amd.virtual_rank(r):
-                t = registry.update_symm_buffer(key, p.view(W, -1)[r])
+                registry.update_symm_buffer(key, p.view(W, -1)[r])
         shard_locals.append(registry.get_symm_buffer(key))
     outs = [torch.empty_like(p) for p in params]
     # register the accumulations up front (lazy registration is not part of a steady-state step)
@@ -220,7 +341,7 @@ def main():
     torch.cuda.synchronize()
 
     comm = get_comm_stream()
-    # One event after every launch of the timed region (plus one at its start): launch k's
+    # One event after every launch of the eager event phase (plus one at its start): launch k's
     # duration is the time between marks k and k+1, all recorded on the launch stream.
     marks = []
 
@@ -229,27 +350,37 @@ def main():
         ev.record(comm)
         marks.append((label, ev))
 
-    def step(i, record):
+    def step(i, record=False):
         m = i % MICROBATCHES
         if m == 0:
             reduction.clear_accumulations()
-            if record and not args.lazy_clear:
+            if record and not reduction.lazy_clear:
                 mark("clear")
         gather.gather_into_tensors(outs, shard_locals, group)
         if record:
             mark("gather")
         reduction.scatter_accumulate_multi(keys, grads[m], group, valid_numels=valid if padded else None)
         if record:
-            mark("store" if m == 0 and args.lazy_clear else "accum")
+            mark("store" if m == 0 and reduction.lazy_clear else "accum")
+
+    def check_against(host_outs, host_accs):
+        ok = True
+        for o, ho in zip(outs, host_outs):
+            ok &= torch.equal(o.cpu().view(torch.int16), ho.view(torch.int16))
+        for key, accs in zip(keys, host_accs):
+            for r, acc in enumerate(reduction.get_peer_accumulations(key)):
+                ok &= torch.equal(acc.cpu().view(torch.int32), accs[r].view(torch.int32))
+        return bool(ok)
 
     # ---- parity + CPU baseline: one full minibatch against the oracle -------------------------
     cpu_baseline = None
     parity = None
+    check_outs = check_accs = None
     if not args.no_verify or not args.no_cpu_baseline:
         from oracle import odc_oracle as oracle
 
         for i in range(MICROBATCHES):
-            step(i, record=False)
+            step(i)
         reduction.sync(group)
         host_params = [p.cpu() for p in params]
         host_grads = [[torch.cat([g.cpu(), torch.zeros(n - g.numel(), dtype=g.dtype)]) if padded else g.cpu()
@@ -257,6 +388,7 @@ def main():
         host_outs = [torch.empty_like(p) for p in host_params]
         host_accs = [[torch.zeros(n // W, dtype=torch.float32) for _ in range(W)] for n in numels]
         host_shards = [list(p.view(W, -1)) for p in host_params]
+
         def cpu_minibatch():
             for m in range(MICROBATCHES):
                 for o, sh in zip(host_outs, host_shards):
@@ -268,6 +400,7 @@ def main():
         cpu_minibatch()  # this first pass also produces the values the GPU is checked against
         first_s = time.perf_counter() - t0
         check_accs = [[a.clone() for a in accs] for accs in host_accs]
+        check_outs = host_outs
         cpu_s, passes = first_s, 1
         if not args.no_cpu_baseline:
             while cpu_s < args.cpu_seconds:  # bounded sample: about 10 s of CPU work
@@ -275,72 +408,109 @@ def main():
                 cpu_minibatch()
                 cpu_s += time.perf_counter() - t0
                 passes += 1
-        host_accs = check_accs
-        cpu_baseline = {
-            "value": round(passes * MICROBATCHES * 14 * N / cpu_s / 1e9, 3),
-            "unit": "GB/s",
-            "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"{passes} x {MICROBATCHES} microbatches of the same layer (gather + "
-                      f"scatter-accumulate) through the torch CPU oracle, {cpu_s:.1f} s",
-        }
-        if args.no_cpu_baseline:
-            cpu_baseline = None
+            cpu_baseline = {
+                "value": round(passes * MICROBATCHES * 14 * N / cpu_s / 1e9, 3),
+                "unit": "GB/s",
+                "cores": torch.get_num_threads(),
+                "kind": "port",
+                "sample": f"{passes} x {MICROBATCHES} microbatches of the same layer (gather + "
+                          f"scatter-accumulate) through the torch CPU oracle, {cpu_s:.1f} s",
+            }
         if not args.no_verify:
-            ok = True
-            for o, ho in zip(outs, host_outs):
-                ok &= torch.equal(o.cpu().view(torch.int16), ho.view(torch.int16))
-            for key, accs in zip(keys, host_accs):
-                for r, acc in enumerate(reduction.get_peer_accumulations(key)):
-                    ok &= torch.equal(acc.cpu().view(torch.int32), accs[r].view(torch.int32))
-            parity = bool(ok)
-            if not ok:
-                print("PARITY FAILURE: GPU results differ from the CPU oracle", file=sys.stderr)
-        del host_params, host_grads, host_outs, host_accs, host_shards
+            parity = check_against(check_outs, check_accs)
+            if not parity:
+                print("PARITY FAILURE: GPU results differ from the CPU oracle (eager launches)", file=sys.stderr)
+        del host_params, host_grads, host_accs, host_shards
 
-    # ---- timed region -----------------------------------------------------------------------
-    # The services launch on the caller's current stream. The timed loop runs on a side stream
-    # of its own (not torch's default stream), and the events are recorded on that same stream,
-    # so that each pair of events brackets exactly one kernel.
-    # A full Python garbage collection (tens of ms with torch imported) landing inside the timed
-    # loop would stall the launches while an event pair is open: collect now, then keep the
-    # collector off until the loop is done.
+    # ---- headline: exactly --steps steps -------------------------------------------------------
+    # A full Python garbage collection (tens of ms with torch imported) landing inside a timed
+    # loop would stall the launches: collect now, then keep the collector off until the end.
     gc.collect()
     gc.disable()
-    with torch.cuda.stream(comm):
-        for i in range(args.warmup):
-            step(i, record=False)
+    full, rest = divmod(args.steps, MICROBATCHES)
+    graph_mb = graph_rest = None
+    if not args.no_graph:
+        # one graph per whole minibatch, one for the steps left over (both start with the clear)
         torch.cuda.synchronize()
-        host_step = []
-        mark("start")
+        graph_mb = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph_mb):
+            for i in range(MICROBATCHES):
+                step(i)
+        if rest:
+            graph_rest = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph_rest):
+                for i in range(rest):
+                    step(i)
+        torch.cuda.synchronize()
+
+    def run_steps(n_full, n_rest):
+        if args.no_graph:
+            for i in range(n_full * MICROBATCHES + n_rest):
+                step(i)
+        else:
+            for _ in range(n_full):
+                graph_mb.replay()
+            if n_rest:
+                graph_rest.replay()
+
+    with torch.cuda.stream(comm):
+        run_steps(-(-args.warmup // MICROBATCHES), 0)  # whole minibatches, at least --warmup steps
+        if rest:
+            run_steps(0, rest)
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
-            ts = time.perf_counter()
-            step(i, record=True)
-            host_step.append(time.perf_counter() - ts)
+        run_steps(full, rest)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
-        if os.environ.get("ODC_BENCH_DEBUG"):
-            print("host ms per step:", [round(x * 1e3, 3) for x in host_step], file=sys.stderr)
-        # the same steps once more in the other clear mode (no events): a secondary figure
+        if not args.no_graph and not args.no_verify and check_accs is not None:
+            # the graphs must leave what the eager launches left: replay one minibatch and compare
+            graph_mb.replay()
+            torch.cuda.synchronize()
+            graph_parity = check_against(check_outs, check_accs)
+            if not graph_parity:
+                print("PARITY FAILURE: graph replay differs from the CPU oracle", file=sys.stderr)
+            parity = bool(parity and graph_parity)
+
+        # ---- eager event phase: per-kernel durations ------------------------------------------
+        for i in range(MICROBATCHES):
+            step(i)
+        torch.cuda.synchronize()
+        mark("start")
+        for i in range(max(args.event_steps, 1)):
+            step(i, record=True)
+        torch.cuda.synchronize()
+
+        # the same steps once more, eagerly, in the other clear mode (no events): a secondary figure
         other = None
         if args.steps >= MICROBATCHES:
+            graph_mb = graph_rest = None  # destroyed: nothing replays into the accumulations any more
+            reduction.forget_captured_graphs()
             reduction.lazy_clear = not args.lazy_clear
             for i in range(MICROBATCHES):
-                step(i, record=False)
+                step(i)
             torch.cuda.synchronize()
             t1 = time.perf_counter()
             for i in range(args.steps):
-                step(i, record=False)
+                step(i)
             torch.cuda.synchronize()
             other_elapsed = time.perf_counter() - t1
             stores = len(range(0, args.steps, MICROBATCHES)) if reduction.lazy_clear else 0
             other_bytes = 14 * N * args.steps - 4 * N * stores
             other = {"clear": "lazy (store on the first microbatch)" if reduction.lazy_clear else "eager",
-                     "value": round(other_bytes / other_elapsed / 1e9, 1), "unit": "GB/s",
+                     "launch": "eager", "value": round(other_bytes / other_elapsed / 1e9, 1), "unit": "GB/s",
                      "bytes_per_step": round(other_bytes / args.steps),
                      "minibatch_ms": round(other_elapsed / args.steps * MICROBATCHES * 1e3, 4)}
             reduction.lazy_clear = args.lazy_clear
+            reduction.clear_accumulations()
+            reduction.sync(group)
+
+    host_overhead = None
+    if not args.no_host_overhead and not padded:
+        host_overhead = measure_host_overhead(torch, odc_amd, comm, group, gather, reduction, registry, outs,
+                                              shard_locals, keys, grads[0], numels, W)
+    ceiling = None
+    if not args.no_ceiling:
+        ceiling = measure_ceiling(torch, comm, N)
     gc.enable()
 
     if args.calibrate:
@@ -356,24 +526,29 @@ def main():
     def mean_ms(label):
         return statistics.fmean(durations[label]) if durations[label] else None
 
-    def measured_traffic(kernel):
-        return MEASURED_TRAFFIC_BYTES.get((kernel, args.layout, W)) if args.workload == "layer" else None
-
+    traffic = load_traffic(args, W)
     g_ms, a_ms, c_ms, s_ms = mean_ms("gather"), mean_ms("accum"), mean_ms("clear"), mean_ms("store")
-    if os.environ.get("ODC_BENCH_DEBUG"):
-        print("gather ms per launch:", [round(x, 3) for x in durations["gather"]], file=sys.stderr)
-        print("accum ms per launch:", [round(x, 3) for x in durations["accum"]], file=sys.stderr)
     accum_gbps = 10 * N / (a_ms * 1e-3) / 1e9
     gather_gbps = 4 * N / (g_ms * 1e-3) / 1e9
     # bytes the timed steps move by the algorithm: a store step's scatter moves 6N, not 10N
-    step_bytes = (14 * N * args.steps - 4 * N * len(durations["store"])) / args.steps
+    timed_stores = len(range(0, args.steps, MICROBATCHES)) if args.lazy_clear else 0
+    step_bytes = (14 * N * args.steps - 4 * N * timed_stores) / args.steps
     value = args.steps * step_bytes / elapsed / 1e9
+    clears = 0 if args.lazy_clear else full + (1 if rest else 0)
+    kernel_sum_ms = None
+    if c_ms is not None or args.lazy_clear:
+        accum_like = a_ms * (args.steps - timed_stores) + (s_ms or 0.0) * timed_stores
+        kernel_sum_ms = (g_ms * args.steps + accum_like + (c_ms or 0.0) * clears) / args.steps
     workload = (f"cfg2: Llama-3-8B decoder layer ({N} bf16 params, {len(keys)} tensors, "
                 f"{args.layout}), W={W} virtual shards, {MICROBATCHES} microbatches per minibatch")
     if args.workload == "uneven":
         workload = (f"cfg3: {len(keys)} flat bf16 parameters of log-uniform size ({sum(valid)} elements, "
                     f"{N} with the zero padding of the shards), none divisible by W={W}, "
                     f"{MICROBATCHES} microbatches per minibatch")
+    if ceiling is not None:
+        ceiling = dict(ceiling)
+        ceiling["accum_frac_of_rmw_ceiling"] = round(accum_gbps / ceiling["rmw_bf16_f32"], 4)
+        ceiling["gather_frac_of_copy_ceiling"] = round(gather_gbps / ceiling["copy"], 4)
     result = {
         "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for gather + scatter-accum, 8B layer, W=8",
         "value": round(value, 1),
@@ -389,8 +564,13 @@ def main():
         "data": "synthetic",
         "config": {"workload": workload, "world_size": W, "elements": N,
                    "bytes_per_step": round(step_bytes), "layout": args.layout,
-                   "clear": "lazy (store on the first microbatch)" if args.lazy_clear else "eager"},
+                   "clear": "lazy (store on the first microbatch)" if args.lazy_clear else "eager",
+                   "launch": "eager" if args.no_graph else
+                             f"HIP graph replay ({full} x one minibatch of {MICROBATCHES} steps"
+                             + (f" + one graph of {rest} steps)" if rest else ")"),
+                   "clears_in_timed_region": clears},
         "frac_of_peak": round(value / HBM_PEAK_GBPS, 4),
+        "kernel_sum_ms_per_step": round(kernel_sum_ms, 4) if kernel_sum_ms else None,
         "roofline": {
             "kernel": "accum_kernel<bf16,f32> (scatter-accumulate)",
             "bound": "hbm",
@@ -398,11 +578,14 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(accum_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("accum"),
+            "traffic": traffic.get("accum", (None, None))[0],
+            "traffic_source": traffic.get("accum", (None, None))[1],
             "algorithmic_bytes": 10 * N,
             "avg_launch_ms": round(a_ms, 5),
             "min_launch_ms": round(min(durations["accum"]), 5),
             "max_launch_ms": round(max(durations["accum"]), 5),
+            "launches_timed": len(durations["accum"]),
+            "practical_ceiling": ceiling,
         },
         "roofline_gather": {
             "kernel": "gather_kernel",
@@ -411,7 +594,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gather_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("gather"),
+            "traffic": traffic.get("gather", (None, None))[0],
+            "traffic_source": traffic.get("gather", (None, None))[1],
             "algorithmic_bytes": 4 * N,
             "avg_launch_ms": round(g_ms, 5),
             "min_launch_ms": round(min(durations["gather"]), 5),
@@ -421,8 +605,9 @@ def main():
                   "GB/s": round(4 * N / (c_ms * 1e-3) / 1e9, 1) if c_ms else None},
         "store": {"avg_launch_ms": round(s_ms, 5) if s_ms else None,
                   "GB/s": round(6 * N / (s_ms * 1e-3) / 1e9, 1) if s_ms else None,
-                  "traffic": measured_traffic("store") if s_ms else None},
+                  "traffic": traffic.get("store", (None, None))[0] if s_ms else None},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 4),
+        "host_us_per_call": host_overhead,
         "other_clear_mode": other,
         "cpu_baseline": cpu_baseline,
         "parity_vs_oracle": parity,

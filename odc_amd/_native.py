@@ -19,6 +19,9 @@ INCLUDE_DIR = _PKG_DIR.parent / "include"
 # $ODC_HIP_LIBRARY points at a library built elsewhere (same ABI); default: the in-tree build
 LIB_PATH = Path(os.environ["ODC_HIP_LIBRARY"]) if os.environ.get("ODC_HIP_LIBRARY") else CSRC_DIR / "libodc_hip.so"
 SOURCES = [CSRC_DIR / "odc_hip.hip"]
+# measurement-only companion: bare streaming kernels that bench.py times as the practical ceiling
+CEILING_LIB_PATH = CSRC_DIR / "libodc_ceiling.so"
+CEILING_SOURCES = [CSRC_DIR / "ceiling_kernels.hip"]
 
 # every symbol include/odc_hip.h declares
 EXPORTED_SYMBOLS = (
@@ -121,7 +124,7 @@ class Span(ctypes.Structure):
     _fields_ = [("offset", ctypes.c_uint64), ("nbytes", ctypes.c_uint64)]
 
 
-def hipcc_command(output: Path = LIB_PATH) -> list[str]:
+def hipcc_command(output: Path = LIB_PATH, sources=None) -> list[str]:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     return [
         hipcc,
@@ -138,13 +141,11 @@ def hipcc_command(output: Path = LIB_PATH) -> list[str]:
         f"-I{INCLUDE_DIR}",
         "-o",
         str(output),
-        *[str(s) for s in SOURCES],
+        *[str(s) for s in (SOURCES if sources is None else sources)],
     ]
 
 
-def build_library(verbose: bool = False) -> Path:
-    """Compile libodc_hip.so in-tree for gfx950 (works without a GPU)."""
-    cmd = hipcc_command()
+def _run_hipcc(cmd, verbose: bool) -> None:
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or proc.returncode != 0:
         print(" ".join(cmd))
@@ -152,7 +153,34 @@ def build_library(verbose: bool = False) -> Path:
         print(proc.stderr)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed with exit code {proc.returncode}")
+
+
+def build_library(verbose: bool = False) -> Path:
+    """Compile libodc_hip.so in-tree for gfx950 (works without a GPU)."""
+    _run_hipcc(hipcc_command(), verbose)
     return LIB_PATH
+
+
+def build_ceiling_library(verbose: bool = False) -> Path:
+    """Compile libodc_ceiling.so (bench.py's bare streaming kernels) in-tree for gfx950."""
+    _run_hipcc(hipcc_command(CEILING_LIB_PATH, CEILING_SOURCES), verbose)
+    return CEILING_LIB_PATH
+
+
+def load_ceiling() -> ctypes.CDLL:
+    """The measurement-only ceiling kernels; built on first use when missing."""
+    if not CEILING_LIB_PATH.exists():
+        build_ceiling_library()
+    lib = ctypes.CDLL(str(CEILING_LIB_PATH))
+    vp, u64, u32, ci = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int
+    P = ctypes.POINTER
+    lib.odc_ceiling_read.argtypes = [vp, u64, vp, ci, u32, vp, P(u64)]
+    lib.odc_ceiling_write.argtypes = [vp, u64, ci, u32, vp, P(u64)]
+    lib.odc_ceiling_copy.argtypes = [vp, vp, u64, ci, u32, vp, P(u64)]
+    lib.odc_ceiling_rmw.argtypes = [vp, vp, u64, ci, u32, vp, P(u64)]
+    for name in ("odc_ceiling_read", "odc_ceiling_write", "odc_ceiling_copy", "odc_ceiling_rmw"):
+        getattr(lib, name).restype = ci
+    return lib
 
 
 _lib = None

@@ -36,6 +36,7 @@
 #include <string>
 
 #include "odc_hip.h"
+#include "odc_tiles.h"
 
 namespace {
 
@@ -103,138 +104,80 @@ int64_t* option_slot(const char* name) {
 // ------------------------------------------------------------------------------------------------
 // device side
 // ------------------------------------------------------------------------------------------------
-#ifndef ODC_TILE_THREADS
-#define ODC_TILE_THREADS 256  // 4 wavefronts of 64 lanes
-#endif
-#ifndef ODC_TILE_UNROLL
-#define ODC_TILE_UNROLL 4  // independent 16 B accesses per lane per stream before the stores
-#endif
-#ifndef ODC_BODY_ALIGN
-#define ODC_BODY_ALIGN 128  // bytes: alignment of a segment's vector body on the written side
-#endif
-constexpr int kThreads = ODC_TILE_THREADS;
-constexpr int kUnroll = ODC_TILE_UNROLL;
-constexpr int kMaxItems = ODC_MAX_ITEMS_PER_LAUNCH;
-constexpr uint32_t kTileVecs = kThreads * kUnroll;      // 16 B vectors per tile
-constexpr uint32_t kTileBytes = kTileVecs * 16;         // gather / clear: 16 KiB of destination
-constexpr uint32_t kTileElems = kTileVecs * 4;          // accumulate: 4096 elements
+using namespace odc_tiles;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Per-launch descriptors, passed by value (kernel argument segment, scalar loads). Every launch
-// carries a TileTable: item i owns tiles [tile_prefix[i], tile_prefix[i+1]), which are
-// world * tiles_per_seg[i] tiles, one run of tiles_per_seg[i] per rank segment.
-struct TileTable {
-  uint32_t world;
-  uint32_t n_items;
-  uint32_t n_tiles;
-  uint32_t rank_major;
-  uint32_t first_rank;
-  uint32_t tile_prefix[kMaxItems + 1];
-  uint32_t tiles_per_seg[kMaxItems];
+// Per-launch descriptors, passed by value (kernel argument segment, scalar loads): the launch's
+// TileTable (odc_tiles.h) and one small record per item.
+struct GatherDesc {
+  uint8_t* dst;
+  uint64_t src_off;
+  uint64_t seg_bytes;
 };
-
 struct GatherLaunch {
   TileTable tt;
-  const uint8_t* base;   // arena base (rank 0 region)
+  const uint8_t* base;  // arena base (rank 0 region)
   uint64_t rank_stride;
-  uint8_t* dst[kMaxItems];
-  uint64_t src_off[kMaxItems];
-  uint64_t seg_bytes[kMaxItems];
+  GatherDesc item[kMaxItems];
 };
 
+struct CastGatherDesc {
+  uint8_t* dst;
+  uint64_t src_off;
+  uint64_t seg_elems;
+};
 struct CastGatherLaunch {
   TileTable tt;
   const uint8_t* base;
   uint64_t rank_stride;
-  uint8_t* dst[kMaxItems];
-  uint64_t src_off[kMaxItems];
-  uint64_t seg_elems[kMaxItems];
+  CastGatherDesc item[kMaxItems];
 };
 
+struct AccumDesc {
+  const uint8_t* grad;
+  uint64_t grad_elems;
+  uint64_t acc_off;
+  uint64_t seg_elems;
+};
 struct AccumLaunch {
   TileTable tt;
   uint8_t* base;
   uint64_t rank_stride;
-  const uint8_t* grad[kMaxItems];
-  uint64_t grad_elems[kMaxItems];
-  uint64_t acc_off[kMaxItems];
-  uint64_t seg_elems[kMaxItems];
+  AccumDesc item[kMaxItems];
 };
 
+struct ClearDesc {
+  uint64_t off;
+  uint64_t seg_bytes;
+};
 struct ClearLaunch {
   TileTable tt;
   uint8_t* base;
   uint64_t rank_stride;
-  uint64_t off[kMaxItems];
-  uint64_t seg_bytes[kMaxItems];
+  ClearDesc item[kMaxItems];
 };
 
+struct PublishDesc {
+  uint8_t* out;  // may be null: divide in place only
+  uint64_t acc_off;
+  uint64_t seg_elems;
+};
 struct PublishLaunch {  // one rank's region only: tt.world == 1
   TileTable tt;
   uint8_t* region;      // base of the publishing rank's region
   float divisor;
   float reciprocal;     // exact 1 / divisor when divide == 2
   uint32_t divide;      // 0: leave the accumulation untouched, 1: divide, 2: multiply by reciprocal
-  uint8_t* out[kMaxItems];  // may be null: divide in place only
-  uint64_t acc_off[kMaxItems];
-  uint64_t seg_elems[kMaxItems];
+  PublishDesc item[kMaxItems];
 };
+static_assert(sizeof(GatherLaunch) <= 4096 && sizeof(AccumLaunch) <= 4096 && sizeof(PublishLaunch) <= 4096 &&
+                  sizeof(CastGatherLaunch) <= 4096 && sizeof(ClearLaunch) <= 4096,
+              "launch descriptors must fit the kernel-argument segment");
 
-// Tile t of a launch -> (item, rank, chunk-in-segment). Everything here is wave-uniform.
-struct TileCoord {
-  uint32_t item, rank, chunk;
-};
-
-__device__ __forceinline__ TileCoord locate_tile(const TileTable& tt, uint32_t t) {
-  TileCoord c;
-  if (tt.rank_major == 2) {
-    // rank outermost: rank r's segments of all items, then rank r+1's. The arena side of the
-    // launch then walks one rank region from item to item. tile_prefix[i] is world times the
-    // tiles before item i within one rank, so the search compares against lt * world.
-    const uint32_t per_rank = tt.n_tiles / tt.world;
-    c.rank = t / per_rank;
-    const uint64_t lt = (uint64_t)(t - c.rank * per_rank) * tt.world;
-    uint32_t lo = 0, hi = tt.n_items;
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (tt.tile_prefix[mid] <= lt) lo = mid; else hi = mid;
-    }
-    c.item = lo;
-    c.chunk = (uint32_t)((lt - tt.tile_prefix[lo]) / tt.world);
-  } else {
-    uint32_t lo = 0, hi = tt.n_items;  // largest i with tile_prefix[i] <= t
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (tt.tile_prefix[mid] <= t) lo = mid; else hi = mid;
-    }
-    const uint32_t lt = t - tt.tile_prefix[lo];
-    const uint32_t tps = tt.tiles_per_seg[lo];
-    c.item = lo;
-    if (tt.rank_major) {
-      c.rank = lt / tps;
-      c.chunk = lt - c.rank * tps;
-    } else {
-      c.chunk = lt / tt.world;
-      c.rank = lt - c.chunk * tt.world;
-    }
-  }
-  c.rank += tt.first_rank;
-  if (c.rank >= tt.world) c.rank -= tt.world;
-  return c;
-}
-
-// Tile geometry shared by all streaming kernels. A rank segment of `n` units (bytes, or
-// elements) whose written side starts at address D is cut as
-//     head  : the units before the first 128-byte line boundary of D (at most 127 bytes),
-//     body  : nvec whole vectors, written with aligned 128-bit (64-bit for 16-bit outputs) stores,
-//     tail  : what is left after the last whole vector.
-// Tile c owns body vectors [c*kTileVecs, (c+1)*kTileVecs); tile 0 also does the head, and the
-// tile holding the last body vector (tile 0 when there is none) the tail. The READ side takes
-// whatever misalignment that leaves it with: gfx950 global loads accept any address, and the
-// typedefs below tell the compiler so. Uneven shards therefore run the same unrolled code as
-// aligned ones; only head, tail and the last partial tile take guarded accesses.
+// The read side of a tile takes whatever misalignment the written side's alignment leaves it
+// with; these typedefs tell the compiler so.
 typedef u32x4 u32x4_u __attribute__((aligned(1)));
 typedef u32x2 u32x2_u __attribute__((aligned(1)));
 
@@ -247,46 +190,19 @@ __device__ __forceinline__ V load_stream(const uint8_t* p) {  // nontemporal, an
   return __builtin_nontemporal_load(reinterpret_cast<const typename Unaligned<V>::type*>(p));
 }
 
-struct SegShape {
-  uint32_t head;   // units before the first line boundary of the written side (clipped to the segment)
-  uint32_t tail;   // units after the last whole vector
-  uint64_t nvec;   // whole vectors
-  uint64_t last;   // tile that owns the tail
-};
-
-// unit_bytes: size of one unit; vec_units: units per vector (vec_units * unit_bytes is 8 or 16)
-__device__ __forceinline__ SegShape seg_shape(uintptr_t written_addr, uint64_t n, uint32_t unit_bytes,
-                                              uint32_t vec_units) {
-  // The body starts on a 128 B line of the written side, not merely on a vector boundary: a
-  // wavefront's 64 vector stores then cover whole lines, none shared with the next wavefront.
-  // (The head is at most 127 bytes, i.e. fewer units than a workgroup has lanes.)
-  constexpr uint32_t kLine = ODC_BODY_ALIGN;
-  static_assert(kLine >= 16 && kLine - 1 <= kThreads, "one lane per head unit");
-  SegShape g;
-  uint64_t head = ((kLine - (uint32_t)(written_addr & (kLine - 1))) & (kLine - 1)) / unit_bytes;
-  if (head > n) head = n;
-  g.head = (uint32_t)head;
-  g.nvec = (n - head) / vec_units;
-  g.tail = (uint32_t)((n - head) - g.nvec * vec_units);
-  g.last = g.nvec ? (g.nvec - 1) / kTileVecs : 0;
-  return g;
-}
-
 // ---- gather -------------------------------------------------------------------------------
 // Everything of a tile that is not a run of kTileVecs whole vectors: the last partial run, the
 // head and the tail. Kept out of line so that the streaming loop stays tight.
-__device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t* s, uint32_t chunk,
-                                                       SegShape g) {
+__device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t* s, uint32_t chunk, SegShape g) {
   // Every load of the tile is issued before its first store (a lone resident workgroup would
   // otherwise pay one memory round trip per step).
   const uint32_t tid = threadIdx.x;
-  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
-  const bool run = v0 < g.nvec && v0 + kTileVecs > g.nvec;
-  const uint32_t left = run ? (uint32_t)(g.nvec - v0) : 0u;
-  const uint8_t* sb = s + g.head + v0 * 16;
-  u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
-  const bool do_head = chunk == 0 && tid < g.head;
-  const bool do_tail = chunk == g.last && tid < g.tail;
+  const TileWork w = tile_work(chunk, g);
+  const uint32_t left = is_whole(w) ? 0u : w.nv;
+  const uint8_t* sb = s + g.head + w.v0 * 16;
+  u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + w.v0;
+  const bool do_head = w.head && tid < g.head;
+  const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 16 + tid;
   u32x4 v[kUnroll];
   uint8_t head_byte = 0, tail_byte = 0;
@@ -302,31 +218,28 @@ __device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t
   if (do_tail) d[tail_at] = tail_byte;
 }
 
-// True when tile `chunk` of a segment has anything besides whole runs of vectors to do.
-__device__ __forceinline__ bool has_edges(uint32_t chunk, const SegShape& g) {
-  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
-  return (v0 < g.nvec && v0 + kTileVecs > g.nvec) || (chunk == 0 && g.head) || (chunk == g.last && g.tail);
-}
-
 __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
   const uint32_t tid = threadIdx.x;
+  TileCursor cur;
+  TileCoord c;
+  GatherDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch.tt, t);
-    const uint64_t seg = launch.seg_bytes[c.item];
-    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.src_off[c.item];
-    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg;
+    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    const uint64_t seg = it.seg_bytes;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + it.src_off;
+    uint8_t* d = it.dst + (uint64_t)c.rank * seg;
     const SegShape g = seg_shape((uintptr_t)d, seg, 1, 16);
-    const uint64_t v0 = (uint64_t)c.chunk * kTileVecs;
-    if (v0 + kTileVecs <= g.nvec) {
-      const uint8_t* sb = s + g.head + (v0 + tid) * 16;
-      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0 + tid;
+    const TileWork w = tile_work(c.chunk, g);
+    if (is_whole(w)) {
+      const uint8_t* sb = s + g.head + (w.v0 + tid) * 16;
+      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + w.v0 + tid;
       u32x4 v[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) v[u] = load_stream<u32x4>(sb + (size_t)u * kThreads * 16);
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], db + u * kThreads);
     }
-    if (has_edges(c.chunk, g)) gather_edges(d, s, c.chunk, g);
+    if (has_edges(w)) gather_edges(d, s, c.chunk, g);
   }
 }
 
@@ -335,33 +248,34 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
 __device__ __attribute__((noinline)) void clear_edges(uint8_t* d, uint32_t chunk, SegShape g) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
   const uint32_t tid = threadIdx.x;
-  const uint64_t v0 = (uint64_t)chunk * kTileVecs;
-  if (v0 < g.nvec && v0 + kTileVecs > g.nvec) {
-    const uint32_t left = (uint32_t)(g.nvec - v0);
-    u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0;
+  const TileWork w = tile_work(chunk, g);
+  if (!is_whole(w)) {
+    u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + w.v0;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      if (u * kThreads + tid < left) db[u * kThreads + tid] = zero;
+      if (u * kThreads + tid < w.nv) db[u * kThreads + tid] = zero;
   }
-  if (chunk == 0 && tid < g.head) d[tid] = 0;
-  if (chunk == g.last && tid < g.tail) d[g.head + g.nvec * 16 + tid] = 0;
+  if (w.head && tid < g.head) d[tid] = 0;
+  if (w.tail && tid < g.tail) d[g.head + g.nvec * 16 + tid] = 0;
 }
 
 __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launch) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
   const uint32_t tid = threadIdx.x;
+  TileCursor cur;
+  TileCoord c;
+  ClearDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch.tt, t);
-    const uint64_t seg = launch.seg_bytes[c.item];
-    uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.off[c.item];
-    const SegShape g = seg_shape((uintptr_t)d, seg, 1, 16);
-    const uint64_t v0 = (uint64_t)c.chunk * kTileVecs;
-    if (v0 + kTileVecs <= g.nvec) {
-      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + v0 + tid;
+    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + it.off;
+    const SegShape g = seg_shape((uintptr_t)d, it.seg_bytes, 1, 16);
+    const TileWork w = tile_work(c.chunk, g);
+    if (is_whole(w)) {
+      u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + w.v0 + tid;
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) db[u * kThreads] = zero;
     }
-    if (has_edges(c.chunk, g)) clear_edges(d, c.chunk, g);
+    if (has_edges(w)) clear_edges(d, c.chunk, g);
   }
 }
 
@@ -459,14 +373,14 @@ __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_
   typedef typename Codec<A>::raw_t araw_t;
   constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
   const uint32_t tid = threadIdx.x;
-  const uint64_t q0 = (uint64_t)chunk * kTileVecs;
-  const uint64_t left = body && q0 < g.nvec ? g.nvec - q0 : 0;
-  const uint64_t e0 = g.head + q0 * 4;
+  const TileWork w = tile_work(chunk, g);
+  const uint32_t left = body ? w.nv : 0u;
+  const uint64_t e0 = g.head + w.v0 * 4;
   avec_t* ap = reinterpret_cast<avec_t*>(acc + e0 * kAB);
   const graw_t* gs = reinterpret_cast<const graw_t*>(grad);
   araw_t* as = reinterpret_cast<araw_t*>(acc);
-  const bool do_head = chunk == 0 && tid < g.head;
-  const bool do_tail = chunk == g.last && tid < g.tail;
+  const bool do_head = w.head && tid < g.head;
+  const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 4 + tid;
 
   float gf[kUnroll][4];
@@ -519,19 +433,21 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
   typedef typename Quad<A>::vec_t avec_t;
   constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
   const uint32_t tid = threadIdx.x;
+  TileCursor cur;
+  TileCoord c;
+  AccumDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch.tt, t);
-    const uint64_t seg = launch.seg_elems[c.item];
-    const uint64_t grad_elems = launch.grad_elems[c.item];
-    const uint8_t* grad = launch.grad[c.item];
-    uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.acc_off[c.item];
+    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    const uint64_t seg = it.seg_elems;
+    uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + it.acc_off;
     const uint64_t g_seg = (uint64_t)c.rank * seg;  // gradient index of the segment's first element
     const SegShape g = seg_shape((uintptr_t)acc, seg, kAB, 4);
-    const uint64_t q0 = (uint64_t)c.chunk * kTileVecs;  // first quad of this tile
-    const uint64_t e0 = g.head + q0 * 4;                // its first element within the segment
-    const bool whole = q0 + kTileVecs <= g.nvec && g_seg + e0 + kTileElems <= grad_elems;
+    const TileWork w = tile_work(c.chunk, g);
+    const uint64_t e0 = g.head + w.v0 * 4;  // the tile's first body element within the segment
+    // whole: all kTileVecs quads exist in the accumulation AND in the valid part of the gradient
+    const bool whole = is_whole(w) && g_seg + e0 + kTileElems <= it.grad_elems;
     if (whole) {
-      const uint8_t* gb = grad + (g_seg + e0) * kGB + (size_t)tid * sizeof(gvec_t);
+      const uint8_t* gb = it.grad + (g_seg + e0) * kGB + (size_t)tid * sizeof(gvec_t);
       avec_t* ap = reinterpret_cast<avec_t*>(acc + e0 * kAB) + tid;
       gvec_t graw[kUnroll];
       avec_t araw[kUnroll];
@@ -551,8 +467,8 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
         __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * kThreads);
       }
     }
-    if (!whole || (c.chunk == 0 && g.head) || (c.chunk == g.last && g.tail))
-      accum_edges<G, A, kStore>(acc, grad, g_seg, grad_elems, c.chunk, g, !whole);
+    if (!whole ? (w.nv != 0 || w.head || w.tail) : (w.head || w.tail))
+      accum_edges<G, A, kStore>(acc, it.grad, g_seg, it.grad_elems, c.chunk, g, !whole);
   }
 }
 
@@ -567,15 +483,15 @@ __device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* 
   typedef typename Codec<D>::raw_t draw_t;
   constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
   const uint32_t tid = threadIdx.x;
-  const uint64_t q0 = (uint64_t)chunk * kTileVecs;
-  const uint64_t left = q0 < g.nvec && q0 + kTileVecs > g.nvec ? g.nvec - q0 : 0;
-  const uint64_t e0 = g.head + q0 * 4;
+  const TileWork w = tile_work(chunk, g);
+  const uint32_t left = is_whole(w) ? 0u : w.nv;
+  const uint64_t e0 = g.head + w.v0 * 4;
   const uint8_t* sb = s + e0 * kSB;
   dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB);
   const sraw_t* ss = reinterpret_cast<const sraw_t*>(s);
   draw_t* ds = reinterpret_cast<draw_t*>(d);
-  const bool do_head = chunk == 0 && tid < g.head;
-  const bool do_tail = chunk == g.last && tid < g.tail;
+  const bool do_head = w.head && tid < g.head;
+  const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 4 + tid;
   // every load of the tile before its first store
   svec_t raw[kUnroll];
@@ -606,15 +522,18 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
   typedef typename Quad<D>::vec_t dvec_t;
   constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
   const uint32_t tid = threadIdx.x;
+  TileCursor cur;
+  TileCoord c;
+  CastGatherDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch.tt, t);
-    const uint64_t seg = launch.seg_elems[c.item];
-    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + launch.src_off[c.item];
-    uint8_t* d = launch.dst[c.item] + (uint64_t)c.rank * seg * kDB;
+    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    const uint64_t seg = it.seg_elems;
+    const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + it.src_off;
+    uint8_t* d = it.dst + (uint64_t)c.rank * seg * kDB;
     const SegShape g = seg_shape((uintptr_t)d, seg, kDB, 4);
-    const uint64_t q0 = (uint64_t)c.chunk * kTileVecs;
-    if (q0 + kTileVecs <= g.nvec) {
-      const uint64_t e0 = g.head + q0 * 4;
+    const TileWork w = tile_work(c.chunk, g);
+    if (is_whole(w)) {
+      const uint64_t e0 = g.head + w.v0 * 4;
       const uint8_t* sb = s + e0 * kSB + (size_t)tid * sizeof(svec_t);
       dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB) + tid;
       svec_t raw[kUnroll];
@@ -627,7 +546,7 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
         __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * kThreads);
       }
     }
-    if (has_edges(c.chunk, g)) cast_edges<S, D>(d, s, c.chunk, g);
+    if (has_edges(w)) cast_edges<S, D>(d, s, c.chunk, g);
   }
 }
 
@@ -641,12 +560,15 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
   typedef typename Quad<A>::vec_t avec_t;
   typedef typename Quad<O>::vec_t ovec_t;
   const uint32_t tid = threadIdx.x;
+  TileCursor cur;
+  TileCoord c;
+  PublishDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    const TileCoord c = locate_tile(launch.tt, t);
-    const uint64_t seg = launch.seg_elems[c.item];
+    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    const uint64_t seg = it.seg_elems;
     const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
-    araw_t* acc = reinterpret_cast<araw_t*>(launch.region + launch.acc_off[c.item]) + in_seg;
-    oraw_t* out = launch.out[c.item] ? reinterpret_cast<oraw_t*>(launch.out[c.item]) + in_seg : nullptr;
+    araw_t* acc = reinterpret_cast<araw_t*>(launch.region + it.acc_off) + in_seg;
+    oraw_t* out = it.out ? reinterpret_cast<oraw_t*>(it.out) + in_seg : nullptr;
     const uint64_t left = seg - in_seg;
     if (left >= kTileElems && (((uintptr_t)acc) & (sizeof(avec_t) - 1)) == 0 &&
         (((uintptr_t)out) & (sizeof(ovec_t) - 1)) == 0) {
@@ -784,8 +706,6 @@ uint32_t lds_claim_for(const odc_arena* a, int64_t cap, uint32_t grid, uint32_t 
   const uint64_t per_wg = ((uint64_t)a->lds_per_cu / (uint64_t)cap) & ~(uint64_t)1023;
   return (uint32_t)std::min<uint64_t>(per_wg, (uint64_t)a->lds_per_wg_max);
 }
-
-constexpr uint64_t kMaxTilesPerLaunch = 1ull << 31;
 
 }  // namespace
 
@@ -995,37 +915,15 @@ int dtype_bytes(int dt) {
   }
 }
 
-// Cuts items [*next, n_items) into one launch: at most kMaxItems non-empty items and fewer than
-// kMaxTilesPerLaunch tiles. units(i) is the item's per-rank size in tile units (0 = skip);
-// take(slot, i) copies item i's descriptor into slot `slot` of the launch. Returns the number of
-// items taken (0 when only empty items were left) or a negative status.
+// odc_tiles::fill_tile_table with its failure turned into an error message.
 template <class Units, class Take>
-int fill_tile_table(TileTable& tt, uint32_t world, uint32_t n_items, uint32_t* next,
-                    uint64_t tile_units, Units units, Take take) {
-  uint32_t n = 0;
-  uint64_t tiles = 0;
-  uint32_t i = *next;
-  for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
-    const uint64_t sz = units(i);
-    if (sz == 0) continue;
-    const uint64_t tps = (sz + tile_units - 1) / tile_units;
-    if (tps * world >= kMaxTilesPerLaunch)
-      return fail(ODC_ERR_INVALID, "item %u: %llu units per rank is too large for one launch", i,
-                  (unsigned long long)sz);
-    if (tiles + tps * world >= kMaxTilesPerLaunch) break;
-    tt.tile_prefix[n] = (uint32_t)tiles;
-    tt.tiles_per_seg[n] = (uint32_t)tps;
-    take(n, i);
-    tiles += tps * world;
-    ++n;
-  }
-  *next = i;
-  for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) tt.tile_prefix[k] = (uint32_t)tiles;
-  for (uint32_t k = n; k < (uint32_t)kMaxItems; ++k) tt.tiles_per_seg[k] = 1;
-  tt.world = world;
-  tt.n_items = n;
-  tt.n_tiles = (uint32_t)tiles;
-  return (int)n;
+int fill_launch(TileTable& tt, uint32_t world, uint32_t n_items, uint32_t* next, uint64_t tile_units,
+                Units units, Take take) {
+  const int n = fill_tile_table(tt, world, n_items, next, tile_units, units, take);
+  if (n < 0)
+    return fail(ODC_ERR_INVALID, "item %d: %llu units per rank is too large for one launch", -1 - n,
+                (unsigned long long)units((uint32_t)(-1 - n)));
+  return n;
 }
 
 int check_rank_range(const odc_arena* a, const char* what, uint32_t i, uint64_t offset, uint64_t nbytes) {
@@ -1111,20 +1009,18 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
     GatherLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = (uint32_t)opt.rank_major;
+    L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
-    const int n = fill_tile_table(
+    const int n = fill_launch(
         L.tt, a->world, n_items, &next, kTileBytes, [&](uint32_t i) { return items[i].shard_bytes; },
         [&](uint32_t slot, uint32_t i) {
-          L.dst[slot] = static_cast<uint8_t*>(items[i].dst);
-          L.src_off[slot] = items[i].src_offset;
-          L.seg_bytes[slot] = items[i].shard_bytes;
+          L.item[slot] = {static_cast<uint8_t*>(items[i].dst), items[i].src_offset, items[i].shard_bytes};
         });
     if (n < 0) return n;
     if (n == 0) continue;
     bool ragged = false;
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
-      ragged |= (((uintptr_t)L.dst[k] | L.src_off[k] | L.seg_bytes[k]) & 15u) != 0;
+      ragged |= (((uintptr_t)L.item[k].dst | L.item[k].src_off | L.item[k].seg_bytes) & 15u) != 0;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles, ragged);
     hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles),
                        static_cast<hipStream_t>(stream), L);
@@ -1162,14 +1058,12 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     CastGatherLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = (uint32_t)opt.rank_major;
+    L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
-    const int n = fill_tile_table(
+    const int n = fill_launch(
         L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
         [&](uint32_t slot, uint32_t i) {
-          L.dst[slot] = static_cast<uint8_t*>(items[i].dst);
-          L.src_off[slot] = items[i].src_offset;
-          L.seg_elems[slot] = items[i].shard_elems;
+          L.item[slot] = {static_cast<uint8_t*>(items[i].dst), items[i].src_offset, items[i].shard_elems};
         });
     if (n < 0) return n;
     if (n == 0) continue;
@@ -1193,13 +1087,12 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
     ClearLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = 0u;  // a write-only stream runs fastest with the ranks interleaved
+    L.tt.order = kRanksInterleaved;  // a write-only stream runs fastest with the ranks interleaved
     L.tt.first_rank = 0;
-    const int n = fill_tile_table(
+    const int n = fill_launch(
         L.tt, a->world, n_spans, &next, kTileBytes, [&](uint32_t i) { return spans[i].nbytes; },
         [&](uint32_t slot, uint32_t i) {
-          L.off[slot] = spans[i].offset;
-          L.seg_bytes[slot] = spans[i].nbytes;
+          L.item[slot] = {spans[i].offset, spans[i].nbytes};
         });
     if (n < 0) return n;
     if (n == 0) continue;
@@ -1252,15 +1145,13 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     AccumLaunch L;
     L.base = a->base;
     L.rank_stride = a->rank_stride;
-    L.tt.rank_major = (uint32_t)opt.rank_major;
+    L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = 0;
-    const int n = fill_tile_table(
+    const int n = fill_launch(
         L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
         [&](uint32_t slot, uint32_t i) {
-          L.grad[slot] = static_cast<const uint8_t*>(items[i].grad);
-          L.grad_elems[slot] = items[i].grad_elems;
-          L.acc_off[slot] = items[i].acc_offset;
-          L.seg_elems[slot] = items[i].shard_elems;
+          L.item[slot] = {static_cast<const uint8_t*>(items[i].grad), items[i].grad_elems, items[i].acc_offset,
+                          items[i].shard_elems};
         });
     if (n < 0) return n;
     if (n == 0) continue;
@@ -1271,9 +1162,9 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     // keeping contiguous once segments get short (measured: +2.3 % at W=64, +5.7 % on 40 uneven
     // parameters at W=12, -0.8 % on the layer at W=8, whose segments average 740 tiles).
     if (opt.accum_tile_order == 3)
-      L.tt.rank_major = (uint64_t)L.tt.n_tiles < 512ull * L.tt.n_items * a->world ? 2u : 1u;
+      L.tt.order = (uint64_t)L.tt.n_tiles < 512ull * L.tt.n_items * a->world ? kRankOutermost : kItemMajor;
     else
-      L.tt.rank_major = (uint32_t)opt.accum_tile_order;
+      L.tt.order = (uint32_t)opt.accum_tile_order;
     // The persistent shape (one workgroup per CU) streams fastest, but only while every rank's
     // chunk of the gradient and of the accumulation starts on a 128 B line: with nothing else
     // resident to cover for it, a workgroup whose wavefronts straddle lines, or that meets heads,
@@ -1283,9 +1174,9 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     // run 2 % faster one workgroup per tile.)
     bool ragged = !(gb == 2 && ab == 4);
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
-      ragged |= (L.acc_off[k] & 127u) != 0 || ((L.seg_elems[k] * ab) & 127u) != 0 ||
-                ((L.seg_elems[k] * gb) & 127u) != 0 || ((uintptr_t)L.grad[k] & 127u) != 0 ||
-                L.grad_elems[k] != L.seg_elems[k] * a->world;
+      ragged |= (L.item[k].acc_off & 127u) != 0 || ((L.item[k].seg_elems * ab) & 127u) != 0 ||
+                ((L.item[k].seg_elems * gb) & 127u) != 0 || ((uintptr_t)L.item[k].grad & 127u) != 0 ||
+                L.item[k].grad_elems != L.item[k].seg_elems * a->world;
     const uint32_t grid =
         grid_for(a, store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
     const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
@@ -1353,14 +1244,12 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
       L.reciprocal = 1.0f / divisor;
       L.divide = 2;
     }
-    L.tt.rank_major = 1u;
+    L.tt.order = kItemMajor;
     L.tt.first_rank = 0;
-    const int n = fill_tile_table(
+    const int n = fill_launch(
         L.tt, 1u, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].elems; },
         [&](uint32_t slot, uint32_t i) {
-          L.out[slot] = static_cast<uint8_t*>(items[i].out);
-          L.acc_off[slot] = items[i].acc_offset;
-          L.seg_elems[slot] = items[i].elems;
+          L.item[slot] = {static_cast<uint8_t*>(items[i].out), items[i].acc_offset, items[i].elems};
         });
     if (n < 0) return n;
     if (n == 0) continue;

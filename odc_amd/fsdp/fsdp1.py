@@ -236,18 +236,23 @@ def pre_optimizer_step(fsdp_module):
     divisor = factor if factor is not None and factor > 1 else 1.0  # `_div_if_needed`
     # a unit that never saw a gradient (frozen, or unused so far) has no accumulation yet
     handles = [h for h in fsdp_module._all_handles if id(h.flat_param) in service.accumulation_indices]
-    by_dtype = {}
+    by_dtype = {}  # one publish launch per (accumulation dtype, parameter dtype)
     for handle in handles:
-        by_dtype.setdefault(handle.flat_param.dtype, []).append(handle)
+        pair = (service.accumulation_dtype_of(id(handle.flat_param)), handle.flat_param.dtype)
+        by_dtype.setdefault(pair, []).append(handle)
     published = set()
-    for dtype, group in by_dtype.items():
+    for (_acc_dtype, dtype), group in by_dtype.items():
         keys = [id(h.flat_param) for h in group]
         for handle, grad in zip(group, service.publish(keys, out_dtype=dtype, divisor=divisor)):
             handle.flat_param.grad = grad
         published.update(keys)
-    rest = [k for k in service.accumulations if k not in published]
-    if rest and divisor != 1.0:  # the reference divides every accumulation, handle or not
-        service.publish(rest, divisor=divisor)
+    if divisor != 1.0:  # the reference divides every accumulation, handle or not (fsdp1.py:324-327)
+        rest = {}
+        for key in service.accumulation_keys:
+            if key not in published:
+                rest.setdefault(service.accumulation_dtype_of(key), []).append(key)
+        for keys in rest.values():
+            service.publish(keys, divisor=divisor)
 
 
 def pre_minibatch_start(_fsdp_module):

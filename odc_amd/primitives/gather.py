@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import logging
+import threading
 from typing import Sequence
 
 from torch import Tensor
@@ -28,9 +29,17 @@ from odc_amd.primitives.utils import (
 logger = logging.getLogger(__name__)
 
 
+class _GatherPlan:
+    """The cached part of one gather call: its item array with everything but the output
+    pointers filled in."""
+
+    __slots__ = ("items", "n", "cast", "src_code", "dst_code", "out_numels")
+
+
 class GatherService:
     def __init__(self):
         self.buffer_splitter = BufferSplitter()
+        self._plans = threading.local()  # per host thread: plan key -> _GatherPlan
 
     def gather_into_tensor(self, output_tensor: Tensor, input_tensor: Tensor, pg) -> None:
         """``output_tensor.view(W, -1)[r] = rank r's copy of input_tensor`` for every r.
@@ -48,56 +57,74 @@ class GatherService:
         dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)
         get_world()  # raises when there is no arena (no GPU, or init_nvshmem not called)
-        registry = SymmBufferRegistry.get_instance()
-        pairs = [(o, i) for o, i in zip(output_tensors, input_tensors) if i.numel() or o.numel()]
-        if not pairs:
+        if any(not i.numel() and not o.numel() for o, i in zip(output_tensors, input_tensors)):
+            pairs = [(o, i) for o, i in zip(output_tensors, input_tensors) if i.numel() or o.numel()]
+            output_tensors, input_tensors = [o for o, _ in pairs], [i for _, i in pairs]
+        if not len(input_tensors):
             return
-        for _, inp in pairs:
+        registry = SymmBufferRegistry.get_instance()
+        src_dtype = input_tensors[0].dtype
+        for inp in input_tensors:
             assert inp.is_cuda and inp.is_contiguous(), "shards are contiguous GPU tensors"
-            assert inp.dtype == pairs[0][1].dtype, "one launch takes one dtype pair"
+            assert inp.dtype == src_dtype, "one launch takes one dtype pair"
         self._gather(
-            [o for o, _ in pairs],
-            [registry.symmetric_offset_of(i) for _, i in pairs],
-            [i.numel() for _, i in pairs],
-            pairs[0][1].dtype,
+            output_tensors,
+            [registry.symmetric_offset_of(i) for i in input_tensors],
+            [i.numel() for i in input_tensors],
+            src_dtype,
             pg,
         )
 
     def _gather(self, outs, src_offsets, shard_numels, src_dtype, pg) -> None:
         """One launch (per 64 items): ``outs[k].view(W, -1)[r]`` = the ``shard_numels[k]`` elements
-        of ``src_dtype`` at symmetric byte offset ``src_offsets[k]`` of rank r."""
+        of ``src_dtype`` at symmetric byte offset ``src_offsets[k]`` of rank r. The item array is
+        built once per (offsets, sizes, dtypes) and host thread; later calls only rewrite the
+        output pointers."""
         world = get_world()
         W = group_size(pg)
         assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
         dst_dtype = outs[0].dtype
-        cast = src_dtype != dst_dtype
-        es = src_dtype.itemsize
-        items = ((_native.GatherCastItem if cast else _native.GatherItem) * len(outs))()
-        for item, out, offset, n in zip(items, outs, src_offsets, shard_numels):
+        cache = getattr(self._plans, "cache", None)
+        if cache is None:
+            cache = self._plans.cache = {}
+        plan_key = (tuple(src_offsets), tuple(shard_numels), src_dtype, dst_dtype)
+        plan = cache.get(plan_key)
+        if plan is None:
+            plan = cache[plan_key] = _GatherPlan()
+            plan.n = len(outs)
+            plan.cast = src_dtype != dst_dtype
+            plan.items = ((_native.GatherCastItem if plan.cast else _native.GatherItem) * plan.n)()
+            plan.out_numels = [W * n for n in shard_numels]
+            es = src_dtype.itemsize
+            for item, offset, n in zip(plan.items, src_offsets, shard_numels):
+                item.src_offset = offset
+                if plan.cast:
+                    item.shard_elems = n
+                else:
+                    item.shard_bytes = n * es
+            # shards kept in one dtype (fp32 master copies), full parameter wanted in another
+            # (bf16): converted on the way instead of gathered and then cast
+            # (odc/fsdp/fsdp1.py:199-223, odc/fsdp/fsdp2.py:341-343)
+            plan.src_code = native_dtype(src_dtype) if plan.cast else None
+            plan.dst_code = native_dtype(dst_dtype) if plan.cast else None
+        items = plan.items
+        for item, out, numel in zip(items, outs, plan.out_numels):
             assert out.is_cuda, "gather runs on the GPU only"
             assert out.dtype == dst_dtype, "one launch takes one dtype pair"
             assert out.is_contiguous()
-            assert out.numel() == W * n, f"output numel {out.numel()} != {W} * shard numel {n}"
+            assert out.numel() == numel, f"output numel {out.numel()} != {W} * shard numel {numel // W}"
             item.dst = out.data_ptr()
-            item.src_offset = offset
-            if cast:
-                item.shard_elems = n
-            else:
-                item.shard_bytes = n * es
 
         lib = _native.load()
-        with comm_stream_section(f"odc.gather[{len(items)}]") as comm:
+        with comm_stream_section("odc.gather") as comm:
             stream = ctypes.c_void_p(comm.cuda_stream)
-            if cast:
-                # shards kept in one dtype (fp32 master copies), full parameter wanted in another
-                # (bf16): converted on the way instead of gathered and then cast
-                # (odc/fsdp/fsdp1.py:199-223, odc/fsdp/fsdp2.py:341-343)
+            if plan.cast:
                 status = lib.odc_gather_cast(
-                    world.arena.handle, items, len(items), native_dtype(src_dtype),
-                    native_dtype(dst_dtype), get_rank(), stream,
+                    world.arena.handle, items, plan.n, plan.src_code, plan.dst_code, get_rank(), stream
                 )
             else:
-                status = lib.odc_gather(world.arena.handle, items, len(items), get_rank(), stream)
+                status = lib.odc_gather(world.arena.handle, items, plan.n, get_rank(), stream)
+        if status:
             _native.check(status)
 
     def gather_slices(
@@ -118,11 +145,14 @@ class GatherService:
         """
         assert len(output_tensors) == len(slice_offsets) == len(slice_numels)
         assert input_tensor.is_cuda and input_tensor.is_contiguous()
+        if not len(output_tensors):
+            return
         es = input_tensor.element_size()
+        total = input_tensor.numel()
         base = SymmBufferRegistry.get_instance().symmetric_offset_of(input_tensor)
         outs, offsets, numels = [], [], []
         for out, off, n in zip(output_tensors, slice_offsets, slice_numels):
-            assert 0 <= off and off + n <= input_tensor.numel(), "slice leaves the buffer"
+            assert 0 <= off and off + n <= total, "slice leaves the buffer"
             if n or out.numel():
                 outs.append(out)
                 offsets.append(base + off * es)

@@ -8,20 +8,29 @@ reference the caller copies chunk r into a staging buffer on rank r (:649-669), 
 doorbells and the watcher collapse into ``odc_scatter_accumulate`` (include/odc_hip.h): one read
 of the gradient, one read-modify-write of the accumulations.
 
-Clears are lazy by default: ``clear_accumulations`` only notes that every accumulation now counts
-as zero, and the first scatter-accumulate of a key after it runs as ``odc_scatter_store``
-(``acc = +0 + grad``, the accumulation is written but never read). The bits are those of a clear
-followed by an accumulate; per minibatch it saves the clear's 4 bytes per element and the first
-read of the accumulation (4 more). Whatever hands an accumulation out (``get_accumulation``,
-``get_peer_accumulations``, ``publish``) first writes the zeros that are still owed.
-``ReductionService(lazy_clear=False)`` or ``ODC_LAZY_CLEAR=0`` clears eagerly.
+Clears are eager by default, as in the reference: ``clear_accumulations`` zeroes every
+accumulation with one launch. ``ReductionService(lazy_clear=True)`` or ``ODC_LAZY_CLEAR=1`` makes
+them lazy: ``clear_accumulations`` then only notes that every accumulation counts as zero, and the
+first scatter-accumulate of a key after it runs as ``odc_scatter_store`` (``acc = +0 + grad``, the
+accumulation is written but never read). The bits are those of a clear followed by an accumulate;
+per minibatch it saves the clear's 4 bytes per element and the first read of the accumulation
+(4 more). Whatever hands an accumulation out (``accumulations``, ``get_accumulation``,
+``get_peer_accumulations``, ``publish``) first writes the zeros that are still owed; a tensor kept
+from an earlier call is not tracked and, in lazy mode only, shows the previous minibatch's sums
+between a clear and the next accumulate.
+
+Launch plans are cached: the ctypes item array of a call (accumulation offsets, shard sizes) is
+built the first time a list of keys and sizes is seen, per host thread, and later calls only
+rewrite the gradient pointers (the reference caches per key too, :599-600).
 """
 
 from __future__ import annotations
 
+import collections.abc
 import ctypes
 import logging
 import os
+import threading
 from typing import Sequence
 
 import torch
@@ -41,17 +50,59 @@ from odc_amd.primitives.utils import (
 logger = logging.getLogger(__name__)
 
 
+class _LiveAccumulations(collections.abc.Sequence):
+    """``ReductionService.accumulations``: the calling rank's live accumulation tensors in
+    registration order, ``accumulations[accumulation_indices[key]]`` being the buffer of ``key``
+    (the list the reference keeps, scatter_accumulate.py:496,554-555, and that its callers
+    iterate and index: ``odc/fsdp/fsdp1.py:324``, ``examples/reduce_scatter.py:169``). Entries are
+    looked up when read, so they follow the virtual rank the process currently plays, and reading
+    one first writes the zeros a lazy clear still owes it."""
+
+    def __init__(self, service):
+        self._service = service
+
+    def __len__(self):
+        return len(self._service.accumulation_keys)
+
+    def __getitem__(self, index):
+        keys = self._service.accumulation_keys[index]
+        if isinstance(index, slice):
+            return [self._service.get_accumulation(k) for k in keys]
+        return self._service.get_accumulation(keys)
+
+    def __iter__(self):
+        for key in list(self._service.accumulation_keys):
+            yield self._service.get_accumulation(key)
+
+    def __repr__(self):
+        return f"<{len(self)} live accumulations>"
+
+
+class _AccumPlan:
+    """The cached part of one scatter-accumulate call: its item array with everything but the
+    gradient pointers filled in."""
+
+    __slots__ = ("items", "n", "grad_code", "acc_code", "acc_dtype", "max_numels", "tiles_exactly", "keys")
+
+    def __init__(self, n):
+        self.items = (_native.AccumItem * n)()
+        self.n = n
+
+
 class ReductionService:
     def __init__(self, accumulation_dtype=None, lazy_clear=None):
-        self.accumulations = []  # index -> key (tensors come from the registry, per rank)
+        self.accumulation_keys = []  # index -> key, in registration order
+        self.accumulations = _LiveAccumulations(self)  # index -> the calling rank's live tensor
         self.accumulation_indices = {}
         self.accumulation_dtype = accumulation_dtype
         self.dispatched_tasks = 0
         self.buffer_splitter = BufferSplitter()
         if lazy_clear is None:
-            lazy_clear = os.environ.get("ODC_LAZY_CLEAR", "1") != "0"
+            lazy_clear = os.environ.get("ODC_LAZY_CLEAR", "0") == "1"
         self.lazy_clear = bool(lazy_clear)
         self._owed_zero = set()  # keys whose accumulations count as zero but hold stale bytes
+        self._captured = set()  # keys ever accumulated under stream capture: always cleared by a kernel
+        self._plans = threading.local()  # per host thread: plan key -> _AccumPlan
 
     # -- registration ---------------------------------------------------------------------
     @staticmethod
@@ -64,17 +115,19 @@ class ReductionService:
         are created: the fused kernel reads the caller's gradient directly."""
         assert len(output_tensor_shape) == 1
         assert key not in self.accumulation_indices
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                "register accumulation keys before capturing: the zeroing of a new accumulation "
+                "would be recorded into the graph and run on every replay"
+            )
         native_dtype(grad_dtype), native_dtype(reduction_dtype)  # reject unsupported dtypes early
         registry = SymmBufferRegistry.get_instance()
         accumulation_key = self._acc_key(key)
         assert not registry.has_key(accumulation_key)
         registry.allocate_symm_buffer(accumulation_key, tuple(output_tensor_shape), reduction_dtype)
-        self.accumulation_indices[key] = len(self.accumulations)
-        self.accumulations.append(key)
-        if self.lazy_clear:
-            self._owed_zero.add(key)
-        else:
-            self._clear_keys([key])
+        self.accumulation_indices[key] = len(self.accumulation_keys)
+        self.accumulation_keys.append(key)
+        self._clear_keys([key])  # a one-time cost; the buffer never shows arena leftovers
 
     def _clear_keys(self, keys):
         keys = list(keys)
@@ -98,35 +151,64 @@ class ReductionService:
         """Zero every registered accumulation of EVERY virtual rank in one launch
         (``acc.fill_(0)`` per key and per process in the reference, :585-587). Idempotent, so
         each virtual rank may call it; like there, no rank may have started the minibatch's
-        scatter-accumulates before the last clear. Lazy mode launches nothing here."""
-        # under stream capture the clear must be a kernel in the graph, not host-side state
-        if self.lazy_clear and not torch.cuda.is_current_stream_capturing():
-            self._owed_zero.update(self.accumulations)
-        else:
-            self._clear_keys(self.accumulations)
+        scatter-accumulates before the last clear.
+
+        Lazy mode launches nothing here, except for keys that a captured HIP graph accumulates
+        into: a graph replays the read-modify-write form whatever the host has noted since, so
+        those are always cleared by a kernel (captured too, when this call is)."""
+        if not self.lazy_clear or torch.cuda.is_current_stream_capturing():
+            self._clear_keys(self.accumulation_keys)
+            return
+        self._clear_keys([k for k in self.accumulation_keys if k in self._captured])
+        self._owed_zero.update(k for k in self.accumulation_keys if k not in self._captured)
 
     def _settle(self, keys):
         """Write the zeros still owed to ``keys`` (before anything reads or adds into them)."""
+        if self._owed_zero:
+            owed = [k for k in keys if k in self._owed_zero]
+            if owed:
+                self._clear_keys(owed)
+
+    def _under_capture(self, keys) -> bool:
+        """Bookkeeping for a scatter-accumulate issued while the current stream is captured into
+        a HIP graph. What the graph records is replayed as recorded, so the choice between the
+        store form and the read-modify-write form cannot depend on host state: the
+        read-modify-write form is recorded, and the keys are from now on cleared by kernels."""
+        if not torch.cuda.is_current_stream_capturing():
+            return False
         owed = [k for k in keys if k in self._owed_zero]
         if owed:
-            self._clear_keys(owed)
+            raise RuntimeError(
+                f"scatter-accumulate captured while {len(owed)} accumulation(s) still owe the zeros of "
+                "a lazy clear: a clear recorded here would run on every replay. Read them once "
+                "(get_accumulation) or run one eager scatter-accumulate before capturing, or use "
+                "eager clears (lazy_clear=False)."
+            )
+        self._captured.update(keys)
+        return True
 
-    def _launch(self, items, grad_dtype, acc_dtype, store):
-        if not len(items):
+    def forget_captured_graphs(self):
+        """Call after destroying every HIP graph that scatter-accumulates into this service's
+        keys: lazy clears may then skip the clear kernel for them again."""
+        self._captured.clear()
+
+    def _launch(self, items, n, grad_code, acc_code, store):
+        if not n:
             return
         lib = _native.load()
         entry = lib.odc_scatter_store if store else lib.odc_scatter_accumulate
         with comm_stream_section("odc.scatter_store" if store else "odc.scatter_accumulate") as comm:
-            _native.check(
-                entry(
-                    get_world().arena.handle,
-                    items,
-                    len(items),
-                    native_dtype(grad_dtype),
-                    native_dtype(acc_dtype),
-                    ctypes.c_void_p(comm.cuda_stream),
-                )
+            status = entry(
+                get_world().arena.handle, items, n, grad_code, acc_code, ctypes.c_void_p(comm.cuda_stream)
             )
+        if status:
+            _native.check(status)
+
+    def _plan_cache(self):
+        cache = getattr(self._plans, "cache", None)
+        if cache is None:
+            cache = self._plans.cache = {}
+        return cache
 
     # -- the primitive ----------------------------------------------------------------------
     def infer_output_shape(self, input_tensor, pg):
@@ -138,28 +220,15 @@ class ReductionService:
         """``acc_r[key] += input_tensor.view(W, -1)[r]`` for every rank r."""
         self.scatter_accumulate_multi([key], [input_tensor], pg)
 
-    def scatter_accumulate_multi(
-        self, keys: Sequence, input_tensors: Sequence[torch.Tensor], pg, valid_numels=None
-    ) -> None:
-        """Multi-tensor form: all (key, gradient) pairs in ONE launch (per 64 pairs).
-
-        ``valid_numels[i]``, when given, says that only the first so many elements of the
-        padded gradient i exist at ``input_tensors[i]``; the rest read as +0 (the ``F.pad`` of
-        ``odc/fsdp/fsdp1.py:25-38`` without materialising it). Then ``input_tensors[i]`` may be
-        shorter than W * shard and the shard size comes from the registered accumulation.
-        """
-        assert len(keys) == len(input_tensors)
-        world = get_world()
-        W = group_size(pg)
-        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+    def _plan_multi(self, keys, input_tensors, pg, valid_numels, W):
+        """Validate a (keys, gradients) list once and build its item array."""
         registry = SymmBufferRegistry.get_instance()
         grad_dtype = input_tensors[0].dtype
-        items = (_native.AccumItem * len(keys))()
+        plan = _AccumPlan(len(keys))
+        plan.keys = tuple(keys)
         acc_dtype = None
         for i, (key, grad) in enumerate(zip(keys, input_tensors)):
-            assert grad.is_cuda, "scatter-accumulate runs on the GPU only"
             assert grad.dtype == grad_dtype, "one launch takes one gradient dtype"
-            assert grad.is_contiguous()
             if valid_numels is None:
                 shard_shape = self.infer_output_shape(grad, pg)
                 valid = grad.numel()
@@ -179,31 +248,70 @@ class ReductionService:
             ), f"key {key}: registered shard {acc_shape}, gradient implies {shard_shape}"
             assert acc_dtype in (None, this_acc_dtype), "one launch takes one accumulation dtype"
             acc_dtype = this_acc_dtype
-            items[i].grad = grad.data_ptr()
-            items[i].grad_elems = valid
-            items[i].acc_offset = offset
-            items[i].shard_elems = shard_shape[0]
+            plan.items[i].grad_elems = valid
+            plan.items[i].acc_offset = offset
+            plan.items[i].shard_elems = shard_shape[0]
+        plan.grad_code = native_dtype(grad_dtype)
+        plan.acc_code = native_dtype(acc_dtype)
+        plan.acc_dtype = acc_dtype
+        return plan
 
-        # Keys that still count as zero take the store form (no read of the accumulation). A key
-        # listed k times goes into k consecutive launches, so its gradients add up in list order.
-        rounds, times_seen = [], {}
-        for i, key in enumerate(keys):
-            k = times_seen.get(key, 0)
-            times_seen[key] = k + 1
-            if k == len(rounds):
-                rounds.append([])
-            rounds[k].append(i)
-        for k, members in enumerate(rounds):
-            for store in (True, False):
-                picked = [i for i in members if (k == 0 and keys[i] in self._owed_zero) == store]
-                if not picked:
-                    continue
-                part = items
-                if len(picked) != len(items):
+    def scatter_accumulate_multi(
+        self, keys: Sequence, input_tensors: Sequence[torch.Tensor], pg, valid_numels=None
+    ) -> None:
+        """Multi-tensor form: all (key, gradient) pairs in ONE launch (per 64 pairs).
+
+        ``valid_numels[i]``, when given, says that only the first so many elements of the
+        padded gradient i exist at ``input_tensors[i]``; the rest read as +0 (the ``F.pad`` of
+        ``odc/fsdp/fsdp1.py:25-38`` without materialising it). Then ``input_tensors[i]`` may be
+        shorter than W * shard and the shard size comes from the registered accumulation.
+        """
+        n = len(keys)
+        assert n == len(input_tensors)
+        if not n:
+            return
+        world = get_world()
+        W = group_size(pg)
+        assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
+        grad_dtype = input_tensors[0].dtype
+        numels = tuple(t.numel() for t in input_tensors)
+        plan_key = ("multi", tuple(keys), numels, grad_dtype,
+                    None if valid_numels is None else tuple(int(v) for v in valid_numels))
+        cache = self._plan_cache()
+        plan = cache.get(plan_key)
+        if plan is None:
+            plan = cache[plan_key] = self._plan_multi(keys, input_tensors, pg, valid_numels, W)
+        items = plan.items
+        for i, grad in enumerate(input_tensors):
+            assert grad.is_cuda, "scatter-accumulate runs on the GPU only"
+            assert grad.dtype == grad_dtype, "one launch takes one gradient dtype"
+            assert grad.is_contiguous()
+            items[i].grad = grad.data_ptr()
+
+        captured = self._under_capture(keys)
+        duplicates = len(set(keys)) != n
+        if not duplicates and (captured or not self._owed_zero or self._owed_zero.isdisjoint(keys)):
+            self._launch(items, n, plan.grad_code, plan.acc_code, False)  # the steady state
+        else:
+            # Keys that still count as zero take the store form (no read of the accumulation). A
+            # key listed k times goes into k consecutive launches, so its gradients add up in
+            # list order.
+            rounds, times_seen = [], {}
+            for i, key in enumerate(keys):
+                k = times_seen.get(key, 0)
+                times_seen[key] = k + 1
+                if k == len(rounds):
+                    rounds.append([])
+                rounds[k].append(i)
+            for k, members in enumerate(rounds):
+                for store in (True, False):
+                    picked = [i for i in members if (k == 0 and keys[i] in self._owed_zero) == store]
+                    if not picked:
+                        continue
                     part = (_native.AccumItem * len(picked))(*[items[i] for i in picked])
-                self._launch(part, grad_dtype, acc_dtype, store)
-        self._owed_zero.difference_update(keys)
-        self.dispatched_tasks += len(items)
+                    self._launch(part, len(picked), plan.grad_code, plan.acc_code, store)
+            self._owed_zero.difference_update(keys)
+        self.dispatched_tasks += n
 
     def scatter_accumulate_slices(
         self,
@@ -224,50 +332,68 @@ class ReductionService:
         ``[W, sum n_i]`` reduce-scatter input. The key is registered on first use with
         ``accumulation_numel`` elements (default: the end of the last slice).
         """
-        assert len(input_tensors) == len(slice_offsets) == len(slice_numels)
+        n = len(input_tensors)
+        assert n == len(slice_offsets) == len(slice_numels)
+        if not n:
+            return
         world = get_world()
         W = group_size(pg)
         assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
-        registry = SymmBufferRegistry.get_instance()
         grad_dtype = input_tensors[0].dtype
-        if key not in self.accumulation_indices:
-            total = accumulation_numel
-            if total is None:
-                total = max(o + n for o, n in zip(slice_offsets, slice_numels))
-            accum_dtype = accumulation_dtype or self.accumulation_dtype or grad_dtype
-            self.register(key, (total,), grad_dtype, accum_dtype, pg)
-        offset, acc_shape, acc_dtype = registry.offsets[self._acc_key(key)]
-        items = (_native.AccumItem * len(input_tensors))()
-        for i, (grad, off, n) in enumerate(zip(input_tensors, slice_offsets, slice_numels)):
-            assert grad.is_cuda and grad.is_contiguous() and grad.dtype == grad_dtype
-            assert 0 <= off and off + n <= acc_shape[0], "slice leaves the accumulation"
-            assert grad.numel() <= W * n, f"gradient {i} has {grad.numel()} > {W} * {n} elements"
-            items[i].grad = grad.data_ptr()
-            items[i].grad_elems = grad.numel()
-            items[i].acc_offset = offset + off * acc_dtype.itemsize
-            items[i].shard_elems = n
-        store = False
-        if key in self._owed_zero:
+        plan_key = ("slices", key, tuple(slice_offsets), tuple(slice_numels), grad_dtype)
+        cache = self._plan_cache()
+        plan = cache.get(plan_key)
+        if plan is None:
+            registry = SymmBufferRegistry.get_instance()
+            if key not in self.accumulation_indices:
+                total = accumulation_numel
+                if total is None:
+                    total = max(o + m for o, m in zip(slice_offsets, slice_numels))
+                accum_dtype = accumulation_dtype or self.accumulation_dtype or grad_dtype
+                self.register(key, (total,), grad_dtype, accum_dtype, pg)
+            offset, acc_shape, acc_dtype = registry.offsets[self._acc_key(key)]
+            plan = _AccumPlan(n)
+            plan.keys = (key,)
+            plan.max_numels = []
+            for i, (off, m) in enumerate(zip(slice_offsets, slice_numels)):
+                assert 0 <= off and off + m <= acc_shape[0], "slice leaves the accumulation"
+                plan.items[i].acc_offset = offset + off * acc_dtype.itemsize
+                plan.items[i].shard_elems = m
+                plan.max_numels.append(W * m)
             # the store form needs the slices to tile the whole accumulation exactly once
-            spans = sorted((int(o), int(n)) for o, n in zip(slice_offsets, slice_numels) if n)
-            end = 0
-            for o, n in spans:
+            end, tiles = 0, True
+            for o, m in sorted((int(o), int(m)) for o, m in zip(slice_offsets, slice_numels) if m):
                 if o != end:
+                    tiles = False
                     break
-                end = o + n
-            else:
-                store = end == acc_shape[0]
+                end = o + m
+            plan.tiles_exactly = tiles and end == acc_shape[0]
+            plan.grad_code = native_dtype(grad_dtype)
+            plan.acc_code = native_dtype(acc_dtype)
+            plan.acc_dtype = acc_dtype
+            cache[plan_key] = plan
+        items = plan.items
+        for i, grad in enumerate(input_tensors):
+            numel = grad.numel()
+            assert grad.is_cuda and grad.is_contiguous() and grad.dtype == grad_dtype
+            assert numel <= plan.max_numels[i], f"gradient {i} has {numel} > {W} * {slice_numels[i]} elements"
+            items[i].grad = grad.data_ptr()
+            items[i].grad_elems = numel
+        store = False
+        if not self._under_capture(plan.keys) and key in self._owed_zero:
+            store = plan.tiles_exactly
             if store:
                 self._owed_zero.discard(key)
             else:
                 self._settle([key])
-        self._launch(items, grad_dtype, acc_dtype, store)
+        self._launch(items, n, plan.grad_code, plan.acc_code, store)
         self.dispatched_tasks += 1
 
     # -- results ----------------------------------------------------------------------------
     def get_accumulation(self, key):
         """The calling rank's live accumulation buffer (callers mutate it in place,
-        ``odc/fsdp/fsdp2.py:846-847``)."""
+        ``odc/fsdp/fsdp2.py:846-847``). With lazy clears, a tensor kept from an earlier call is
+        not updated by ``clear_accumulations`` until the next accumulate; ask again instead."""
         if key not in self.accumulation_indices:
             raise KeyError(key)
         self._settle([key])
@@ -314,6 +440,10 @@ class ReductionService:
                 )
             )
         return results
+
+    def accumulation_dtype_of(self, key) -> torch.dtype:
+        """The dtype the accumulation of ``key`` was registered with."""
+        return SymmBufferRegistry.get_instance().offsets[self._acc_key(key)][2]
 
     def _registry_peers(self, key):
         """The W accumulation buffers as they are in memory (owed zeros not written)."""

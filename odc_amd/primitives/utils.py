@@ -493,12 +493,11 @@ def _tracing() -> bool:
     return os.environ.get("ODC_TRACE", "0") == "1"
 
 
-@contextlib.contextmanager
-def comm_stream_section(label: str = "odc"):
-    """The stream the body's launches go to. With ``ODC_TRACE=1`` the section is a marker
-    range named ``label`` (roctx through ``torch.cuda.nvtx``; the reference brackets the same
-    places with NVTX, ``scatter_accumulate.py:307,383,736``), visible to
-    ``rocprofv3 --marker-trace``.
+class comm_stream_section:
+    """``with comm_stream_section(label) as stream:`` — the stream the body's launches go to.
+    With ``ODC_TRACE=1`` the section is a marker range named ``label`` (roctx through
+    ``torch.cuda.nvtx``; the reference brackets the same places with NVTX,
+    ``scatter_accumulate.py:307,383,736``), visible to ``rocprofv3 --marker-trace``.
 
     The reference hops to its comm stream and joins it with the current stream on both sides
     (``gather.py:114,176``; ``scatter_accumulate.py:636-640,725-727``), which orders a launch
@@ -507,28 +506,42 @@ def comm_stream_section(label: str = "odc"):
     streams, and on this GPU every extra hardware queue with event joins in flight slows the
     dispatch of all queues (measured on a Llama layer stack: 28.8 -> 22.4 ms per microbatch).
     ``ODC_COMM_STREAM=dedicated`` restores the hop."""
-    traced = _tracing()
-    if traced:
-        torch.cuda.nvtx.range_push(label)
-    try:
-        current = torch.cuda.current_stream()
-        if launch_stream_policy() == "caller":
-            _launch_streams[current.cuda_stream] = current
-            yield current
-            return
-        comm = get_comm_stream()
-        _launch_streams[comm.cuda_stream] = comm
-        if current == comm:
-            yield comm
-            return
-        comm.wait_stream(current)
+
+    __slots__ = ("label", "_traced", "_current", "_comm")
+
+    def __init__(self, label: str = "odc"):
+        self.label = label
+
+    def __enter__(self):
+        self._traced = _tracing()
+        self._comm = None
+        if self._traced:
+            torch.cuda.nvtx.range_push(self.label)
         try:
-            yield comm
+            current = torch.cuda.current_stream()
+            if launch_stream_policy() == "caller":
+                _launch_streams[current.cuda_stream] = current
+                return current
+            comm = get_comm_stream()
+            _launch_streams[comm.cuda_stream] = comm
+            if current == comm:
+                return comm
+            comm.wait_stream(current)
+            self._current, self._comm = current, comm
+            return comm
+        except BaseException:
+            if self._traced:
+                torch.cuda.nvtx.range_pop()
+            raise
+
+    def __exit__(self, exc_type, exc, tb):
+        try:
+            if self._comm is not None:
+                self._current.wait_stream(self._comm)
         finally:
-            current.wait_stream(comm)
-    finally:
-        if traced:
-            torch.cuda.nvtx.range_pop()
+            if self._traced:
+                torch.cuda.nvtx.range_pop()
+        return False
 
 
 def wait_for_launches() -> None:

@@ -60,16 +60,16 @@ def _run_layer(make_world, W, layout, microbatches):
 
 @pytest.mark.parametrize("layout", ["per-param", "flat"])
 def test_config2_llama_layer_w8(make_world, layout):
-    """Llama-3-8B decoder layer, W=8: 9 per-parameter shards in one multi-tensor launch, and the
-    same 218 112 000 elements as one flat shard of 27 264 000."""
-    _run_layer(make_world, 8, layout, microbatches=3)
+    """Llama-3-8B decoder layer, W=8, a minibatch of 8 microbatches: 9 per-parameter shards in one
+    multi-tensor launch, and the same 218 112 000 elements as one flat shard of 27 264 000."""
+    _run_layer(make_world, 8, layout, microbatches=8)
 
 
 @pytest.mark.parametrize("layout", ["per-param", "flat"])
 def test_config4_small_chunks_w64(make_world, layout):
-    """The same layer at W=64: shards from 917 504 elements down to the 64-element (128 B)
-    slices of the two norm vectors."""
-    _run_layer(make_world, 64, layout, microbatches=2)
+    """The same layer at W=64, a minibatch of 16 microbatches: shards from 917 504 elements down to
+    the 64-element (128 B) slices of the two norm vectors."""
+    _run_layer(make_world, 64, layout, microbatches=16)
 
 
 def test_config3_uneven_padded_w12(make_world):
@@ -124,12 +124,13 @@ def test_config5_full_llama3_8b_sweep(make_world):
     scatter-accumulate unit by unit in reverse order. Values come from per-(unit, microbatch) seeded
     device generators, so they can be drawn again for checking:
       * every unit: gathered parameters equal the regenerated parameters; accumulations equal
-        (0 + g0) + g1 computed with torch's fp32 add on the device (an independent implementation);
+        ((0 + g0) + g1) + ... over the 8 microbatches, computed with torch's fp32 add on the device
+        (an independent implementation);
       * sampled units (embedding, two layers, head): bit-exact against the CPU oracle."""
     from odc_amd import virtual_rank
     from odc_amd.workloads import llama3_8b_units
 
-    W, M = 8, 2
+    W, M = 8, 8
     units = llama3_8b_units()
     total = sum(numel(s) for _, unit in units for _, s in unit)
     assert total == 8_030_261_248
@@ -172,16 +173,19 @@ def test_config5_full_llama3_8b_sweep(make_world):
     for u, (_, unit) in enumerate(units):
         for p, (_, shape) in enumerate(unit):
             n = numel(shape)
-            g0, g1 = draw(u, p, 0, n, 1e-3), draw(u, p, 1, n, 1e-3)
-            expect = (torch.zeros(n, device="cuda") + g0.float()) + g1.float()
+            expect = torch.zeros(n, device="cuda")
+            accs = [torch.zeros(n // W) for _ in range(W)] if u in sampled else None
+            for m in range(M):
+                g = draw(u, p, m, n, 1e-3)
+                expect += g.float()
+                if accs is not None:
+                    oracle.scatter_accumulate(accs, g.cpu())
+                del g
             got = torch.cat(list(reduction.get_peer_accumulations((u, p))))
             assert torch.equal(got.view(torch.int32), expect.view(torch.int32)), (u, p)
-            if u in sampled:
-                accs = [torch.zeros(n // W) for _ in range(W)]
-                oracle.scatter_accumulate(accs, g0.cpu())
-                oracle.scatter_accumulate(accs, g1.cpu())
+            if accs is not None:
                 assert_bit_equal(got, torch.cat(accs), f"unit {u} param {p} vs oracle")
-            del g0, g1, expect, got
+            del expect, got
 
 
 @pytest.mark.parametrize("W", [8, 12])

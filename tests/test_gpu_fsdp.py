@@ -13,6 +13,14 @@ from oracle import odc_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["eager", "lazy"], autouse=True)
+def clear_mode(request, monkeypatch):
+    """Every test here runs with the reference's eager clears (the default) and with lazy clears
+    (ODC_LAZY_CLEAR=1, read when the FSDP patches build their ReductionService)."""
+    monkeypatch.setenv("ODC_LAZY_CLEAR", "1" if request.param == "lazy" else "0")
+    return request.param
+
+
 def test_fsdp1_hooks_and_call_sites(make_world):
     """One minibatch the way examples/llm_training/torch_fsdp.py:462-481 drives it:
     pre_minibatch_start, per microbatch gather + reduce_grad for two flat params, then

@@ -17,6 +17,14 @@ from test_gpu_fsdp2_torch import Block, Toy
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["eager", "lazy"], autouse=True)
+def clear_mode(request, monkeypatch):
+    """Every test here runs with the reference's eager clears (the default) and with lazy clears
+    (ODC_LAZY_CLEAR=1, read when the FSDP patches build their ReductionService)."""
+    monkeypatch.setenv("ODC_LAZY_CLEAR", "1" if request.param == "lazy" else "0")
+    return request.param
+
+
 @pytest.fixture
 def fake_process_group():
     from torch.testing._internal.distributed.fake_pg import FakeStore

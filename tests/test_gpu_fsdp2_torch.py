@@ -16,6 +16,14 @@ from oracle import odc_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["eager", "lazy"], autouse=True)
+def clear_mode(request, monkeypatch):
+    """Every test here runs with the reference's eager clears (the default) and with lazy clears
+    (ODC_LAZY_CLEAR=1, read when the FSDP patches build their ReductionService)."""
+    monkeypatch.setenv("ODC_LAZY_CLEAR", "1" if request.param == "lazy" else "0")
+    return request.param
+
+
 class Block(nn.Module):
     def __init__(self, dim, hidden):
         super().__init__()

@@ -73,6 +73,8 @@ def test_scatter_store_every_bf16_pattern(make_world):
     red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
     all_bf16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
     red.register("all", (65536 // W,), torch.bfloat16, torch.float32, group)
+    red.clear_accumulations()  # lazy: nothing is launched, the next accumulate stores
+    assert red._owed_zero == {"all"}
     poison(red._registry_peers("all"))
     red.scatter_accumulate("all", all_bf16.cuda(), group)
     want = [torch.zeros(65536 // W) for _ in range(W)]
@@ -101,9 +103,10 @@ def test_lazy_clear_matches_the_oracle(make_world, seed):
     want = {k: [torch.zeros(s, dtype=acc_dtype) for _ in range(W)] for k, s in sizes.items()}
     for k, s in sizes.items():
         lazy.register(k, (s,), grad_dtype, acc_dtype, group)
-    assert lazy._owed_zero == set(sizes)
+    assert not lazy._owed_zero  # registration zeroes eagerly
     for minibatch in range(3):
         lazy.clear_accumulations()
+        assert lazy._owed_zero == set(sizes)
         for k in sizes:
             poison(lazy._registry_peers(k))
             for w in want[k]:
@@ -148,6 +151,7 @@ def test_slices_that_tile_the_accumulation_take_the_store_form(make_world, seed)
     group = make_world(W, 16 << 20)
     red = ReductionService(accumulation_dtype=acc_dtype, lazy_clear=True)
     red.register("g", (total,), grad_dtype, acc_dtype, group)
+    red.clear_accumulations()  # lazy: "g" now owes its zeros
     poison(red._registry_peers("g"))
     g = torch.Generator().manual_seed(seed)
     want = [torch.zeros(total, dtype=acc_dtype) for _ in range(W)]
@@ -192,3 +196,70 @@ def test_clear_stays_eager_under_graph_capture(make_world):
         red.scatter_accumulate("k", grad, group)
         for acc in red.get_peer_accumulations("k"):
             assert_bit_equal(acc, torch.ones(S), f"replay {replay}: one accumulate after the clear")
+
+
+@pytest.mark.parametrize("lazy", [True, False])
+def test_captured_accumulate_with_clears_outside_the_graph(make_world, lazy):
+    """A graph that holds only the scatter-accumulate, replayed M times per minibatch, with
+    clear_accumulations() called OUTSIDE capture between minibatches: the graph always replays
+    the read-modify-write form, so the clear must be a kernel even in lazy mode, and a later
+    get_accumulation must not zero what the replays added."""
+    from odc_amd import ReductionService
+
+    W, S, M = 4, 30_001, 3
+    group = make_world(W, 8 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=lazy)
+    g = torch.Generator().manual_seed(21)
+    grad_host = (torch.randn(W * S, generator=g) * 1e-3).bfloat16()
+    grad = grad_host.cuda()
+    eager_host = (torch.randn(W * S, generator=g) * 1e-3).bfloat16()
+    # warm-up as torch's graph recipe has it: one eager call (registers the key, takes the store
+    # form in lazy mode), then the capture
+    red.clear_accumulations()
+    red.scatter_accumulate("k", grad, group)
+    red.sync(group)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        red.scatter_accumulate("k", grad, group)
+    for minibatch in range(2):
+        red.clear_accumulations()  # outside capture
+        want = [torch.zeros(S) for _ in range(W)]
+        for m in range(M):
+            graph.replay()
+            oracle.scatter_accumulate(want, grad_host)
+            if m == 0:  # eager work of the same key between replays
+                red.scatter_accumulate("k", eager_host.cuda(), group)
+                oracle.scatter_accumulate(want, eager_host)
+            torch.cuda.synchronize()
+        for r, acc in enumerate(red.get_peer_accumulations("k")):
+            assert_bit_equal(acc, want[r], f"minibatch {minibatch}, rank {r}")
+        assert_bit_equal(red.get_accumulation("k"), want[0], f"minibatch {minibatch}: handed out")
+
+
+def test_capture_refuses_an_accumulation_that_owes_zeros(make_world):
+    """Lazy mode: recording the store form (or a clear) into a graph would overwrite the sums on
+    every replay, so a capture that meets owed zeros fails loudly instead."""
+    from odc_amd import ReductionService
+
+    W, S = 4, 4096
+    group = make_world(W, 4 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
+    grad = torch.ones(W * S, dtype=torch.bfloat16, device="cuda")
+    red.scatter_accumulate("k", grad, group)
+    red.clear_accumulations()  # "k" now owes zeros
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="owe the zeros"):
+        with torch.cuda.graph(graph):
+            red.scatter_accumulate("k", grad, group)
+    torch.cuda.synchronize()
+    # registering under capture is refused as well (its zeroing would be recorded)
+    graph2 = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="before capturing"):
+        with torch.cuda.graph(graph2):
+            red.scatter_accumulate("new", grad, group)
+    torch.cuda.synchronize()
+    # the service still works eagerly afterwards
+    red.scatter_accumulate("k", grad, group)
+    assert_bit_equal(red.get_accumulation("k"), torch.ones(S), "store after the refused capture")
