@@ -68,6 +68,8 @@ def parse_args():
                     help="eager steps with one HIP event per launch, for the per-kernel roofline figures")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the bare streaming kernels")
     ap.add_argument("--no-host-overhead", action="store_true", help="skip the host-time-per-call measurement")
+    ap.add_argument("--no-launch-floor", action="store_true",
+                    help="skip the one-tile launches (they would skew a profiler's per-kernel averages)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline sample length")
     ap.add_argument("--no-verify", action="store_true")
@@ -242,6 +244,42 @@ def measure_ceiling(torch, comm, N, iters=12):
                     "rmw 10N, read 4N, write 4N), launched alternately, HIP events per launch"}
 
 
+def measure_launch_floor(torch, comm, group, gather, reduction, registry, W, launches=50):
+    """What a launch costs before any bandwidth: gather and scatter-accumulate of ONE 64-element
+    item (one 128-byte slice per rank, the smallest shard of the layer at W=64), event to event on
+    the launch stream, and the same with the device idle before each launch."""
+    small = registry.allocate_symm_buffer("bench_floor_shard", (64,), torch.bfloat16)
+    out = torch.empty(W * 64, dtype=torch.bfloat16, device="cuda")
+    grad = torch.zeros(W * 64, dtype=torch.bfloat16, device="cuda")
+    reduction.register("bench_floor", (64,), torch.bfloat16, torch.float32, group)
+    result = {}
+    with torch.cuda.stream(comm):
+        for label, fn in (("gather_one_tile", lambda: gather.gather_into_tensor(out, small, group)),
+                          ("scatter_accumulate_one_tile", lambda: reduction.scatter_accumulate("bench_floor", grad, group))):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            events = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+            events[0].record(comm)
+            for k in range(launches):
+                fn()
+                events[k + 1].record(comm)
+            torch.cuda.synchronize()
+            back_to_back = statistics.fmean(a.elapsed_time(b) for a, b in zip(events, events[1:])) * 1e3
+            idle = []
+            for _ in range(launches):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(comm)
+                fn()
+                e1.record(comm)
+                torch.cuda.synchronize()
+                idle.append(e0.elapsed_time(e1) * 1e3)
+            result[label] = {"back_to_back_us": round(back_to_back, 2), "from_idle_us": round(statistics.median(idle), 2)}
+    result["note"] = (f"HIP-event interval per launch of one 64-element item (W x 128 B), mean of {launches} "
+                      "queued launches, and median when the device is idle before each")
+    return result
+
+
 def measure_host_overhead(torch, odc_amd, comm, group, gather, reduction, registry, outs, shard_locals, keys,
                           grads, numels, W, calls=100):
     """Host time of one call, mean over `calls` back-to-back asynchronous calls (the launches
@@ -314,7 +352,7 @@ def main():
     padded = numels != valid
     assert padded == (args.workload == "uneven")
     N = sum(numels)
-    per_rank = sum((n // W) * 12 + 2048 for n in numels) + (1 << 20)  # shards, accumulations, and the same again as one group
+    per_rank = sum((n // W) * 12 + 2048 for n in numels) + (2 << 20)  # shards, accumulations, and the same again as one group
     group = odc_amd.init_nvshmem(world_size=W, symmetric_size=per_rank)
     registry = odc_amd.SymmBufferRegistry.get_instance()
     gather = odc_amd.GatherService()
@@ -508,6 +546,9 @@ def main():
     if not args.no_host_overhead and not padded:
         host_overhead = measure_host_overhead(torch, odc_amd, comm, group, gather, reduction, registry, outs,
                                               shard_locals, keys, grads[0], numels, W)
+    launch_floor = None
+    if not args.no_launch_floor:
+        launch_floor = measure_launch_floor(torch, comm, group, gather, reduction, registry, W)
     ceiling = None
     if not args.no_ceiling:
         ceiling = measure_ceiling(torch, comm, N)
@@ -608,6 +649,7 @@ def main():
                   "traffic": traffic.get("store", (None, None))[0] if s_ms else None},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 4),
         "host_us_per_call": host_overhead,
+        "launch_floor_us": launch_floor,
         "other_clear_mode": other,
         "cpu_baseline": cpu_baseline,
         "parity_vs_oracle": parity,

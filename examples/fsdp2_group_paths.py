@@ -10,6 +10,7 @@ Per operation the reference's data flow (``fused=False``) is timed against the f
     reduce    chunk_cat of bf16 gradients into fp32 [W, sum n_p] + scatter-accumulate
               (odc/fsdp/fsdp2.py:671-682, 708-710)                   vs  one scatter-accumulate
     publish   acc /= W, then acc.to(bf16) (odc/fsdp/fsdp2.py:846-847, 897-899) vs  one pass
+    clear     acc.fill_(0) per rank (odc/primitives/scatter_accumulate.py:585-587) vs  one launch
 
 Both flows are bit-identical (tests/test_gpu_fsdp.py); this script only times them.
 
@@ -32,6 +33,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--world-size", type=int, default=8)
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
     args = ap.parse_args()
 
     import odc_amd as odc
@@ -88,7 +91,14 @@ def main():
         ("reduce (bf16 gradients -> fp32 accumulations)", timed(lambda: layer.reduce(grads, fused=False)),
          timed(lambda: layer.reduce(grads, fused=True)), 10 * N),
         ("publish (acc /= W, bf16 copy; one rank)", timed(publish_reference), timed(publish_fused), 10 * N // W),
+        ("clear (zero the fp32 accumulations of all ranks)", timed(lambda: [a.zero_() for a in scatter.get_peer_accumulations(id(layer))]),
+         timed(scatter.clear_accumulations), 4 * N),
     ]
+    if args.calibrate:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
     print(f"Llama-3-8B layer as one FSDP2 group: {N} parameters, W={W}")
     print(f"{'':48s} {'reference flow':>15s} {'fused':>10s} {'fused GB/s':>11s}")
     for name, ref_ms, fused_ms, fused_bytes in rows:

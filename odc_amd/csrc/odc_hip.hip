@@ -77,6 +77,7 @@ struct Options {
   int64_t store_resident_cap = 4;
   int64_t clear_blocks_per_cu = 0;
   int64_t publish_blocks_per_cu = 0;
+  int64_t publish_resident_cap = 0;
   int64_t rank_major = 1;        // gather: 0 = ranks interleaved, 1 = item-major, 2 = rank outermost
   int64_t accum_tile_order = 3;  // the same for scatter-accumulate / store; 3 = by segment length
   int64_t rank_stagger_bytes = 0;
@@ -98,6 +99,7 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "accum_resident_cap")) return &g_opt.accum_resident_cap;
   if (!strcmp(name, "store_blocks_per_cu")) return &g_opt.store_blocks_per_cu;
   if (!strcmp(name, "store_resident_cap")) return &g_opt.store_resident_cap;
+  if (!strcmp(name, "publish_resident_cap")) return &g_opt.publish_resident_cap;
   return nullptr;
 }
 
@@ -221,10 +223,14 @@ __device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t
 __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
-  TileCoord c;
   GatherDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    if (!cursor_holds(cur, t)) {
+      cursor_seek(launch.tt, t, cur);
+      it = launch.item[cur.item];  // issued together with the loads of cursor_enter
+      cursor_enter(launch.tt, cur);
+    }
+    const TileCoord c = cursor_coord(launch.tt, cur, t);
     const uint64_t seg = it.seg_bytes;
     const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + it.src_off;
     uint8_t* d = it.dst + (uint64_t)c.rank * seg;
@@ -263,10 +269,14 @@ __global__ __launch_bounds__(kThreads) void clear_kernel(const ClearLaunch launc
   const u32x4 zero = {0u, 0u, 0u, 0u};
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
-  TileCoord c;
   ClearDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    if (!cursor_holds(cur, t)) {
+      cursor_seek(launch.tt, t, cur);
+      it = launch.item[cur.item];  // issued together with the loads of cursor_enter
+      cursor_enter(launch.tt, cur);
+    }
+    const TileCoord c = cursor_coord(launch.tt, cur, t);
     uint8_t* d = launch.base + (uint64_t)c.rank * launch.rank_stride + it.off;
     const SegShape g = seg_shape((uintptr_t)d, it.seg_bytes, 1, 16);
     const TileWork w = tile_work(c.chunk, g);
@@ -434,10 +444,14 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
   constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
-  TileCoord c;
   AccumDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    if (!cursor_holds(cur, t)) {
+      cursor_seek(launch.tt, t, cur);
+      it = launch.item[cur.item];  // issued together with the loads of cursor_enter
+      cursor_enter(launch.tt, cur);
+    }
+    const TileCoord c = cursor_coord(launch.tt, cur, t);
     const uint64_t seg = it.seg_elems;
     uint8_t* acc = launch.base + (uint64_t)c.rank * launch.rank_stride + it.acc_off;
     const uint64_t g_seg = (uint64_t)c.rank * seg;  // gradient index of the segment's first element
@@ -523,10 +537,14 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
   constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
-  TileCoord c;
   CastGatherDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    if (!cursor_holds(cur, t)) {
+      cursor_seek(launch.tt, t, cur);
+      it = launch.item[cur.item];  // issued together with the loads of cursor_enter
+      cursor_enter(launch.tt, cur);
+    }
+    const TileCoord c = cursor_coord(launch.tt, cur, t);
     const uint64_t seg = it.seg_elems;
     const uint8_t* s = launch.base + (uint64_t)c.rank * launch.rank_stride + it.src_off;
     uint8_t* d = it.dst + (uint64_t)c.rank * seg * kDB;
@@ -561,10 +579,14 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
   typedef typename Quad<O>::vec_t ovec_t;
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
-  TileCoord c;
   PublishDesc it = {};
   for (uint32_t t = blockIdx.x; t < launch.tt.n_tiles; t += gridDim.x) {
-    if (locate_tile(launch.tt, t, cur, c)) it = launch.item[c.item];
+    if (!cursor_holds(cur, t)) {
+      cursor_seek(launch.tt, t, cur);
+      it = launch.item[cur.item];  // issued together with the loads of cursor_enter
+      cursor_enter(launch.tt, cur);
+    }
+    const TileCoord c = cursor_coord(launch.tt, cur, t);
     const uint64_t seg = it.seg_elems;
     const uint64_t in_seg = (uint64_t)c.chunk * kTileElems;
     araw_t* acc = reinterpret_cast<araw_t*>(launch.region + it.acc_off) + in_seg;
@@ -1255,7 +1277,8 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
     if (n == 0) continue;
     // one workgroup per tile: the division sequence wants the occupancy, and the launch is short
     const uint32_t grid = grid_for(a, opt.publish_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.publish_resident_cap, grid, L.tt.n_tiles),
+                       static_cast<hipStream_t>(stream), L);
     ODC_HIP_TRY(hipGetLastError());
   }
   return ODC_OK;

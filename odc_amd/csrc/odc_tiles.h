@@ -48,70 +48,79 @@ constexpr uint64_t kMaxTilesPerLaunch = 1ull << 31;
 //   kRankOutermost    : rank by rank; within a rank item by item
 enum TileOrder : uint32_t { kRanksInterleaved = 0, kItemMajor = 1, kRankOutermost = 2 };
 
-// Travels by value in the kernel-argument segment. Item i owns tiles
-// [tile_prefix[i], tile_prefix[i+1]) (in the item-major orders), which are
-// world * tiles_per_seg[i] tiles: one run of tiles_per_seg[i] per rank segment. Entries past
-// n_items hold n_tiles, so a search never lands on them.
+// Travels by value in the kernel-argument segment. seg_prefix[i] is the number of tiles that
+// the items before item i have in ONE rank segment each, so item i has
+// seg_prefix[i+1] - seg_prefix[i] tiles per rank segment and world times that in the launch.
+// Entries past n_items hold tiles_per_rank, so a search never lands on them.
 struct TileTable {
   uint32_t world;
   uint32_t n_items;
-  uint32_t n_tiles;
+  uint32_t n_tiles;         // world * tiles_per_rank
   uint32_t order;           // TileOrder
   uint32_t first_rank;      // rotation of the rank walk (never changes the result)
-  uint32_t tiles_per_rank;  // n_tiles / world
-  uint32_t tile_prefix[kMaxItems + 1];
-  uint32_t tiles_per_seg[kMaxItems];
+  uint32_t tiles_per_rank;  // seg_prefix[n_items]
+  uint32_t seg_prefix[kMaxItems + 1];
 };
 
 struct TileCoord {
   uint32_t item, rank, chunk;  // chunk: tile index within the rank segment
 };
 
-// Largest i with tile_prefix[i] <= x, for x < n_tiles (tile_prefix[0] is 0 and the entries are
-// strictly increasing over the real items: empty items are never listed).
-ODC_HD uint32_t find_item(const TileTable& tt, uint64_t x) {
+// Largest i with seg_prefix[i] <= x, for x < tiles_per_rank (seg_prefix[0] is 0 and the entries
+// are strictly increasing over the real items: empty items are never listed).
+ODC_HD uint32_t find_item(const TileTable& tt, uint32_t x) {
   uint32_t lo = 0, hi = tt.n_items;
   while (hi - lo > 1) {
     const uint32_t mid = (lo + hi) >> 1;
-    if (tt.tile_prefix[mid] <= x) lo = mid; else hi = mid;
+    if (tt.seg_prefix[mid] <= x) lo = mid; else hi = mid;
   }
   return lo;
 }
 
 // A cursor remembers the run of consecutive tile indices [lo, hi) that share the item (and, in
 // rank-outermost order, the rank) of the last tile located, so a workgroup that walks many tiles
-// with a grid-stride loop searches only when it leaves that run.
+// with a grid-stride loop searches only when it leaves that run. Use:
+//     if (!cursor_holds(cur, t)) {
+//       cursor_seek(tt, t, cur);            // the search: sets cur.item
+//       desc = launch.item[cur.item];       // the caller's per-item record ...
+//       cursor_enter(tt, cur);              // ... and the run's bounds: independent loads
+//     }
+//     TileCoord c = cursor_coord(tt, cur, t);
 struct TileCursor {
   uint32_t lo = 1, hi = 0;  // empty
   uint32_t item = 0;
   uint32_t rank = 0;  // kRankOutermost only: the (unrotated) rank of the run
-  uint32_t tps = 1;   // tiles_per_seg[item]
+  uint32_t tps = 1;   // tiles per rank segment of the item
 };
 
-// Tile t of a launch -> (item, rank, chunk). Returns true when the cursor moved to another item
-// (the caller then reloads the item's descriptor). Everything here is wave-uniform.
-ODC_HD bool locate_tile(const TileTable& tt, uint32_t t, TileCursor& cur, TileCoord& c) {
-  bool moved = false;
-  if (t < cur.lo || t >= cur.hi) {
-    moved = true;
-    if (tt.order == kRankOutermost) {
-      // tile_prefix[i] is world times the tiles before item i within one rank
-      const uint32_t rank = t / tt.tiles_per_rank;
-      const uint32_t local = t - rank * tt.tiles_per_rank;
-      const uint32_t i = find_item(tt, (uint64_t)local * tt.world);
-      cur.item = i;
-      cur.rank = rank;
-      cur.tps = tt.tiles_per_seg[i];
-      cur.lo = rank * tt.tiles_per_rank + tt.tile_prefix[i] / tt.world;
-      cur.hi = cur.lo + cur.tps;
-    } else {
-      const uint32_t i = find_item(tt, t);
-      cur.item = i;
-      cur.tps = tt.tiles_per_seg[i];
-      cur.lo = tt.tile_prefix[i];
-      cur.hi = tt.tile_prefix[i + 1];
-    }
+ODC_HD bool cursor_holds(const TileCursor& cur, uint32_t t) { return t >= cur.lo && t < cur.hi; }
+
+ODC_HD void cursor_seek(const TileTable& tt, uint32_t t, TileCursor& cur) {
+  if (tt.order == kRankOutermost) {
+    cur.rank = t / tt.tiles_per_rank;
+    cur.item = find_item(tt, t - cur.rank * tt.tiles_per_rank);
+  } else {
+    // item i owns tiles [seg_prefix[i] * world, seg_prefix[i+1] * world)
+    cur.rank = 0;
+    cur.item = find_item(tt, t / tt.world);
   }
+}
+
+ODC_HD void cursor_enter(const TileTable& tt, TileCursor& cur) {
+  const uint32_t first = tt.seg_prefix[cur.item], next = tt.seg_prefix[cur.item + 1];
+  cur.tps = next - first;
+  if (tt.order == kRankOutermost) {
+    cur.lo = cur.rank * tt.tiles_per_rank + first;
+    cur.hi = cur.lo + cur.tps;
+  } else {
+    cur.lo = first * tt.world;
+    cur.hi = next * tt.world;
+  }
+}
+
+// Tile t (inside the cursor's run) -> (item, rank, chunk). Everything here is wave-uniform.
+ODC_HD TileCoord cursor_coord(const TileTable& tt, const TileCursor& cur, uint32_t t) {
+  TileCoord c;
   const uint32_t lt = t - cur.lo;
   c.item = cur.item;
   if (tt.order == kRankOutermost) {
@@ -126,6 +135,17 @@ ODC_HD bool locate_tile(const TileTable& tt, uint32_t t, TileCursor& cur, TileCo
   }
   c.rank += tt.first_rank;
   if (c.rank >= tt.world) c.rank -= tt.world;
+  return c;
+}
+
+// The three steps in one call. Returns true when the cursor moved to another run.
+ODC_HD bool locate_tile(const TileTable& tt, uint32_t t, TileCursor& cur, TileCoord& c) {
+  const bool moved = !cursor_holds(cur, t);
+  if (moved) {
+    cursor_seek(tt, t, cur);
+    cursor_enter(tt, cur);
+  }
+  c = cursor_coord(tt, cur, t);
   return moved;
 }
 
@@ -194,7 +214,7 @@ template <class Units, class Take>
 inline int fill_tile_table(TileTable& tt, uint32_t world, uint32_t n_items, uint32_t* next,
                            uint64_t tile_units, Units units, Take take) {
   uint32_t n = 0;
-  uint64_t tiles = 0;
+  uint64_t tiles = 0, per_rank = 0;
   uint32_t i = *next;
   for (; i < n_items && n < (uint32_t)kMaxItems; ++i) {
     const uint64_t sz = units(i);
@@ -202,19 +222,18 @@ inline int fill_tile_table(TileTable& tt, uint32_t world, uint32_t n_items, uint
     const uint64_t tps = tiles_for(sz, tile_units);
     if (tps * world >= kMaxTilesPerLaunch) return -1 - (int)i;
     if (tiles + tps * world >= kMaxTilesPerLaunch) break;
-    tt.tile_prefix[n] = (uint32_t)tiles;
-    tt.tiles_per_seg[n] = (uint32_t)tps;
+    tt.seg_prefix[n] = (uint32_t)per_rank;
     take(n, i);
     tiles += tps * world;
+    per_rank += tps;
     ++n;
   }
   *next = i;
-  for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) tt.tile_prefix[k] = (uint32_t)tiles;
-  for (uint32_t k = n; k < (uint32_t)kMaxItems; ++k) tt.tiles_per_seg[k] = 1;
+  for (uint32_t k = n; k <= (uint32_t)kMaxItems; ++k) tt.seg_prefix[k] = (uint32_t)per_rank;
   tt.world = world;
   tt.n_items = n;
   tt.n_tiles = (uint32_t)tiles;
-  tt.tiles_per_rank = world ? (uint32_t)(tiles / world) : 0;
+  tt.tiles_per_rank = (uint32_t)per_rank;
   return (int)n;
 }
 

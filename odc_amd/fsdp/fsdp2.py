@@ -476,21 +476,20 @@ def foreach_reduce(fsdp_params, unsharded_grads, reduce_scatter_group, reduce_sc
     return placeholder, reduce_scatter_event, post_reduce_event, None, None, partial_reduce_output
 
 
-@torch.no_grad()
-def update_gradients(fsdp_param_group) -> None:
-    """fsdp2.py:795-957 for a torch param group: average and post-divide the calling rank's
-    accumulation in place, cast to the parameter dtype, hand the strided views to the sharded
-    parameters as DTensor gradients."""
+def _publish_request(fsdp_param_group):
+    """First half of ``update_gradients`` (fsdp2.py:795-899) for a torch param group: take the
+    group's reduce context and say what the end-of-minibatch pass over its accumulation is, as
+    ``(key, out_dtype, divisor, touched)``; None when no microbatch ran through the group in this
+    minibatch (fsdp2.py:797-801). Whatever cannot be folded into one pass (an all-reduce hook, a
+    separate post-divide: two roundings) is done here."""
     import torch.distributed as dist
     from torch.distributed.fsdp._fully_shard._fsdp_collectives import _get_gradient_divide_factors
-    from torch.distributed.tensor import DTensor
 
     ctx = getattr(fsdp_param_group, "_odc_reduce_context", None)
     if ctx is None:
-        return  # no microbatch ran through this group in this minibatch (fsdp2.py:797-801)
+        return None
     del fsdp_param_group._odc_reduce_context
     touched = fsdp_param_group.__dict__.pop("_odc_params_with_grad", None)
-    layout = _group_layout(fsdp_param_group)
     rs_group = ctx["reduce_scatter_group"]
     _pre, postdivide_factor, reduce_scatter_op, _ar_op = _get_gradient_divide_factors(
         rs_group, None, ctx["reduce_dtype"], ctx["device"].type, ctx["gradient_divide_factor"],
@@ -499,7 +498,7 @@ def update_gradients(fsdp_param_group) -> None:
     assert reduce_scatter_op in (dist.ReduceOp.SUM, dist.ReduceOp.AVG), f"{reduce_scatter_op} is not supported"
     scatter = get_reduction_service()
     key = id(fsdp_param_group)
-    orig_dtype = ctx["orig_dtype"] or scatter.get_accumulation(key).dtype
+    orig_dtype = ctx["orig_dtype"] or scatter.accumulation_dtype_of(key)
     if ctx["all_reduce_hook"] is not None or (postdivide_factor is not None and postdivide_factor > 1):
         # two roundings (average, then post-divide) and a user hook in between
         if reduce_scatter_op == dist.ReduceOp.AVG:
@@ -507,10 +506,17 @@ def update_gradients(fsdp_param_group) -> None:
         if ctx["all_reduce_hook"] is not None:
             ctx["all_reduce_hook"](scatter.get_accumulation(key))
         divisor = postdivide_factor if postdivide_factor is not None and postdivide_factor > 1 else 1.0
-        (reduce_output,) = scatter.publish([key], out_dtype=orig_dtype, divisor=divisor)
     else:
         divisor = float(rs_group.size()) if reduce_scatter_op == dist.ReduceOp.AVG else 1.0
-        (reduce_output,) = scatter.publish([key], out_dtype=orig_dtype, divisor=divisor)
+    return key, orig_dtype, float(divisor), touched
+
+
+def _hand_out_gradients(fsdp_param_group, reduce_output, touched) -> None:
+    """Second half of ``update_gradients`` (fsdp2.py:902-939): strided views of the published
+    shard become the sharded parameters' DTensor gradients."""
+    from torch.distributed.tensor import DTensor
+
+    layout = _group_layout(fsdp_param_group)
     base = reduce_output.storage_offset()
     for fp, off in zip(fsdp_param_group.fsdp_params, layout.offsets):
         if touched is not None and id(fp) not in touched:
@@ -526,6 +532,39 @@ def update_gradients(fsdp_param_group) -> None:
             fp.sharded_param.grad = fp.to_sharded_dtensor(new_sharded_grad)
         for hook in (getattr(fp.sharded_param, "_post_accumulate_grad_hooks", {}) or {}).values():
             hook(fp.sharded_param)
+
+
+@torch.no_grad()
+def update_gradients(fsdp_param_group) -> None:
+    """fsdp2.py:795-957 for one torch param group: average and post-divide the calling rank's
+    accumulation in place, cast to the parameter dtype, hand the strided views to the sharded
+    parameters as DTensor gradients."""
+    request = _publish_request(fsdp_param_group)
+    if request is None:
+        return
+    key, out_dtype, divisor, touched = request
+    (reduce_output,) = get_reduction_service().publish([key], out_dtype=out_dtype, divisor=divisor)
+    _hand_out_gradients(fsdp_param_group, reduce_output, touched)
+
+
+@torch.no_grad()
+def update_all_gradients(fsdp_param_groups) -> None:
+    """``update_gradients`` for every group of a model with as few passes as possible: the
+    groups whose accumulations share (accumulation dtype, gradient dtype, divisor) are divided
+    and cast by ONE launch (per 64 groups) instead of one short launch each."""
+    scatter = get_reduction_service()
+    batches = {}
+    for group in fsdp_param_groups:
+        request = _publish_request(group)
+        if request is None:
+            continue
+        key, out_dtype, divisor, touched = request
+        batches.setdefault((scatter.accumulation_dtype_of(key), out_dtype, divisor), []).append((group, key, touched))
+    for (_acc_dtype, out_dtype, divisor), members in batches.items():
+        outputs = scatter.publish([key for _, key, _ in members], out_dtype=out_dtype, divisor=divisor)
+        for (group, _key, touched), reduce_output in zip(members, outputs):
+            with torch.cuda.nvtx.range(f"update_gradients:{group._module_fqn}"):
+                _hand_out_gradients(group, reduce_output, touched)
 
 
 def _is_torch_fsdp_module(fsdp_module) -> bool:
@@ -550,12 +589,11 @@ def pre_optimizer_step(fsdp_module):
     """fsdp2.py:1023-1046: sync once, then publish every group's gradients."""
     scatter = get_reduction_service()
     if _is_torch_fsdp_module(fsdp_module):
-        for i, group in enumerate(_torch_param_groups(fsdp_module)):
-            if i == 0:
-                with torch.cuda.nvtx.range("scatter_accumulate_sync"):
-                    scatter.sync(group.mesh_info.shard_process_group)
-            with torch.cuda.nvtx.range(f"update_gradients:{group._module_fqn}"):
-                update_gradients(group)
+        groups = _torch_param_groups(fsdp_module)
+        if groups:
+            with torch.cuda.nvtx.range("scatter_accumulate_sync"):
+                scatter.sync(groups[0].mesh_info.shard_process_group)
+            update_all_gradients(groups)
         return
     for i, group in enumerate(_param_groups(fsdp_module)):
         if i == 0:

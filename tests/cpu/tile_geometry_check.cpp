@@ -46,20 +46,22 @@ static const Kind kKinds[] = {
     {2, 4, kTileElems},   // 16-bit accumulations / outputs: 4 elements per 8-byte vector
 };
 
+static uint32_t tiles_per_seg(const TileTable& tt, uint32_t i) { return tt.seg_prefix[i + 1] - tt.seg_prefix[i]; }
+
 // The order's definition, enumerated the slow way: the sequence of (slot, unrotated rank, chunk).
 static std::vector<TileCoord> enumerate_order(const TileTable& tt) {
   std::vector<TileCoord> seq;
   if (tt.order == kRankOutermost) {
     for (uint32_t r = 0; r < tt.world; ++r)
       for (uint32_t i = 0; i < tt.n_items; ++i)
-        for (uint32_t c = 0; c < tt.tiles_per_seg[i]; ++c) seq.push_back({i, r, c});
+        for (uint32_t c = 0; c < tiles_per_seg(tt, i); ++c) seq.push_back({i, r, c});
   } else if (tt.order == kItemMajor) {
     for (uint32_t i = 0; i < tt.n_items; ++i)
       for (uint32_t r = 0; r < tt.world; ++r)
-        for (uint32_t c = 0; c < tt.tiles_per_seg[i]; ++c) seq.push_back({i, r, c});
+        for (uint32_t c = 0; c < tiles_per_seg(tt, i); ++c) seq.push_back({i, r, c});
   } else {
     for (uint32_t i = 0; i < tt.n_items; ++i)
-      for (uint32_t c = 0; c < tt.tiles_per_seg[i]; ++c)
+      for (uint32_t c = 0; c < tiles_per_seg(tt, i); ++c)
         for (uint32_t r = 0; r < tt.world; ++r) seq.push_back({i, r, c});
   }
   return seq;
@@ -80,13 +82,21 @@ static void check_launch(const TileTable& tt0, const std::vector<Item>& slots, c
     for (int gsel = 0; gsel < 4; ++gsel) {
       const uint32_t grid = grids[gsel] < tt.n_tiles ? grids[gsel] : tt.n_tiles;
       for (uint32_t b = 0; b < grid; ++b) {
-        TileCursor cur;
-        TileCoord c;
+        TileCursor cur, cur2;
         uint32_t held_item = ~0u;
         for (uint32_t t = b; t < tt.n_tiles; t += grid) {
-          const bool moved = locate_tile(tt, t, cur, c);
-          if (moved) held_item = c.item;  // what a kernel reloads its descriptor for
+          // exactly the kernels' sequence
+          if (!cursor_holds(cur, t)) {
+            cursor_seek(tt, t, cur);
+            held_item = cur.item;  // what a kernel reloads its descriptor for
+            cursor_enter(tt, cur);
+            REQUIRE(cursor_holds(cur, t), "t %u is outside the run the cursor entered", t);
+          }
+          const TileCoord c = cursor_coord(tt, cur, t);
           REQUIRE(held_item == c.item, "t %u: the cursor changed item without saying so", t);
+          TileCoord c2;
+          locate_tile(tt, t, cur2, c2);
+          REQUIRE(c2.item == c.item && c2.rank == c.rank && c2.chunk == c.chunk, "locate_tile disagrees at t %u", t);
           const uint32_t rot = (want[t].rank + tt.first_rank) % tt.world;
           REQUIRE(c.item == want[t].item && c.rank == rot && c.chunk == want[t].chunk,
                   "order %u first_rank %u grid %u t %u: got (%u,%u,%u) want (%u,%u,%u)", order, tt.first_rank, grid,
@@ -163,9 +173,11 @@ static void run_case(std::mt19937_64& rng, uint32_t world, uint32_t n_items, con
     if (n == 0) continue;
     ++launches;
     REQUIRE(tt.n_items == (uint32_t)n && tt.world == world && tt.tiles_per_rank * world == tt.n_tiles, "table header");
-    for (uint32_t k = 0; k + 1 <= tt.n_items; ++k)
-      REQUIRE(tt.tile_prefix[k + 1] - tt.tile_prefix[k] == tt.tiles_per_seg[k] * world, "prefix %u", k);
-    for (uint32_t k = tt.n_items; k <= (uint32_t)kMaxItems; ++k) REQUIRE(tt.tile_prefix[k] == tt.n_tiles, "padding %u", k);
+    REQUIRE(tt.seg_prefix[0] == 0, "prefix starts at 0");
+    for (uint32_t k = 0; k < tt.n_items; ++k)
+      REQUIRE(tiles_per_seg(tt, k) == tiles_for(slots[k].n, kind.tile_units) && tiles_per_seg(tt, k) > 0, "prefix %u", k);
+    for (uint32_t k = tt.n_items; k <= (uint32_t)kMaxItems; ++k)
+      REQUIRE(tt.seg_prefix[k] == tt.tiles_per_rank, "padding %u", k);
     check_launch(tt, slots, kind, rng);
   }
   uint32_t nonempty = 0;

@@ -40,7 +40,7 @@ def test_the_library_is_built_from_the_checked_header():
     """The kernels must take their geometry from odc_tiles.h, not from a private copy."""
     text = (ROOT / "odc_amd" / "csrc" / "odc_hip.hip").read_text()
     assert '#include "odc_tiles.h"' in text
-    for name in ("locate_tile(", "seg_shape(", "tile_work(", "fill_tile_table("):
+    for name in ("cursor_seek(", "cursor_enter(", "cursor_coord(", "seg_shape(", "tile_work(", "fill_tile_table("):
         assert name in text, name
     for private in ("struct TileTable", "struct SegShape", "TileCoord locate_tile"):
         assert private not in text, f"{private} is defined in odc_hip.hip again"
