@@ -252,6 +252,7 @@ def measure_launch_floor(torch, comm, group, gather, reduction, registry, W, lau
     out = torch.empty(W * 64, dtype=torch.bfloat16, device="cuda")
     grad = torch.zeros(W * 64, dtype=torch.bfloat16, device="cuda")
     reduction.register("bench_floor", (64,), torch.bfloat16, torch.float32, group)
+    torch.cuda.synchronize()
     result = {}
     with torch.cuda.stream(comm):
         for label, fn in (("gather_one_tile", lambda: gather.gather_into_tensor(out, small, group)),
@@ -274,9 +275,26 @@ def measure_launch_floor(torch, comm, group, gather, reduction, registry, W, lau
                 e1.record(comm)
                 torch.cuda.synchronize()
                 idle.append(e0.elapsed_time(e1) * 1e3)
-            result[label] = {"back_to_back_us": round(back_to_back, 2), "from_idle_us": round(statistics.median(idle), 2)}
-    result["note"] = (f"HIP-event interval per launch of one 64-element item (W x 128 B), mean of {launches} "
-                      "queued launches, and median when the device is idle before each")
+            # the same launches replayed from one HIP graph: no host time between them
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(launches):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            g0.record(comm)
+            graph.replay()
+            g1.record(comm)
+            torch.cuda.synchronize()
+            result[label] = {"eager_back_to_back_us": round(back_to_back, 2),
+                             "eager_from_idle_us": round(statistics.median(idle), 2),
+                             "graph_replay_us": round(g0.elapsed_time(g1) * 1e3 / launches, 2)}
+            del graph
+    result["note"] = (f"microseconds per launch of one 64-element item (W x 128 B): HIP-event interval, mean of "
+                      f"{launches} eager launches queued back to back (bounded by the host's time per call), "
+                      "median when the device is idle before each, and per launch when the same "
+                      f"{launches} launches are replayed from one HIP graph (the device-side floor)")
     return result
 
 
