@@ -149,14 +149,23 @@ def main():
     t_plain = timed(unsharded_minibatch, args.steps) / args.microbatches
     tokens = args.batch * args.seq
     layer_params = sum(p.numel() for p in twin.model.layers[0].parameters())
-    # per microbatch and layer: two converting gathers (forward, backward) and one scatter-accumulate
-    path_bytes = args.layers * layer_params * (2 * 6 + 10)
+    # per microbatch: every decoder layer is gathered twice (forward, backward; fp32 shards -> bf16,
+    # 6 B per element) and scatter-accumulated once (10 B); the root group (embedding, final norm,
+    # lm_head) stays unsharded after its forward gather, so it is gathered once
+    root_params = n_params - args.layers * layer_params
+    path_bytes = args.layers * layer_params * (2 * 6 + 10) + root_params * (6 + 10)
     print(f"Llama {args.layers} x ({args.hidden}, {args.intermediate}) + vocab {args.vocab}: {n_params / 1e6:.0f} M parameters, "
           f"W={W}, {tokens} tokens per microbatch")
     print(f"sharded through ODC : {t_sharded * 1e3:8.2f} ms per microbatch  ({tokens / t_sharded:,.0f} tokens/s)")
     print(f"unsharded, same GPU : {t_plain * 1e3:8.2f} ms per microbatch  ({tokens / t_plain:,.0f} tokens/s)")
-    print(f"difference          : {(t_sharded - t_plain) * 1e3:8.2f} ms; the decoder layers' gathers and "
-          f"scatter-accumulates alone move {path_bytes / 1e9:.2f} GB = {path_bytes / 6.2e12 * 1e3:.2f} ms at 6.2 TB/s")
+    t_path = path_bytes / 6.2e12
+    print(f"difference          : {(t_sharded - t_plain) * 1e3:8.2f} ms; the gathers and "
+          f"scatter-accumulates alone move {path_bytes / 1e9:.2f} GB = {t_path * 1e3:.2f} ms at 6.2 TB/s")
+    from odc_amd.primitives.utils import launch_stream_policy
+
+    print(f"hidden behind compute (ODC_COMM_STREAM={launch_stream_policy()}): "
+          f"{max(0.0, 1.0 - (t_sharded - t_plain) / t_path):.0%} of that time "
+          "(1 - difference / path time; FSDP's own bookkeeping counts against it)")
     fsdp2.stop()
     fsdp2.unpatch_fsdp2()
     odc.finalize_distributed()
