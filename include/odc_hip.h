@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define ODC_HIP_ABI_VERSION 1
+#define ODC_HIP_ABI_VERSION 2
 
 typedef enum odc_status {
   ODC_OK = 0,
@@ -54,8 +54,15 @@ typedef struct odc_arena odc_arena;
 
 enum {
   ODC_ARENA_DEVICE = 0,     /* hipMalloc-backed (the product path) */
-  ODC_ARENA_NO_BACKING = 1  /* offsets only, no memory: for sizing an arena before creating it.
+  ODC_ARENA_NO_BACKING = 1, /* offsets only, no memory: for sizing an arena before creating it.
                                Every compute entry point refuses it with ODC_ERR_NO_BACKING. */
+  ODC_ARENA_DRY_RUN = 2     /* no memory and no GPU needed: the compute entry points validate their
+                               arguments, split the work list and plan every launch against a
+                               fictitious base address, then count the launch instead of issuing it
+                               (odc_get_option "dry_run_launches" / "dry_run_tiles" /
+                               "dry_run_workgroups"; odc_set_option("dry_run_reset", 0) zeroes them).
+                               For testing the host side of the library without a device; implies
+                               ODC_ARENA_NO_BACKING for odc_arena_ptr / odc_arena_locate. */
 };
 
 typedef struct odc_arena_info {
@@ -207,7 +214,7 @@ int odc_abi_version(void);
 /* Launch-shape knobs, for measurement. "gather_blocks_per_cu", "accum_blocks_per_cu",
  * "store_blocks_per_cu", "clear_blocks_per_cu", "publish_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
  * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
- * "cast_resident_cap", "accum_resident_cap", "store_resident_cap": for one-workgroup-per-tile
+ * "cast_resident_cap", "accum_resident_cap", "store_resident_cap", "publish_resident_cap": for one-workgroup-per-tile
  * launches, the most workgroups resident per CU
  * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather; "accum_tile_order" for
  * scatter-accumulate and scatter-store: 1 = walk a rank's whole shard before the next rank, item by

@@ -45,7 +45,7 @@ EXPORTED_SYMBOLS = (
     "odc_get_option",
 )
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 MAX_ITEMS_PER_LAUNCH = 64
 
 ODC_OK = 0
@@ -58,6 +58,7 @@ ODC_ERR_NO_BACKING = -6
 
 ODC_ARENA_DEVICE = 0
 ODC_ARENA_NO_BACKING = 1
+ODC_ARENA_DRY_RUN = 2
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1

@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -659,7 +660,9 @@ struct odc_arena {
   int lds_per_wg_max = 64 * 1024;
   uint64_t bytes_per_rank = 0;
   uint64_t rank_stride = 0;
-  uint8_t* base = nullptr;
+  uint8_t* base = nullptr;    // the hipMalloc (null without backing)
+  uint8_t* origin = nullptr;  // what launches are planned against: base, or a fictitious address on a dry-run arena
+  bool dry_run = false;
   std::map<uint64_t, uint64_t> live;  // offset -> size (rounded)
   std::map<uint64_t, uint64_t> free_; // offset -> size, coalesced
   uint64_t in_use = 0;
@@ -700,9 +703,31 @@ class DeviceGuard {
 
 int check_compute(odc_arena* a, DeviceGuard& guard) {
   if (int rc = check_arena(a)) return rc;
+  if (a->dry_run) return ODC_OK;  // plans against a fictitious address, launches nothing
   if (!a->base)
     return fail(ODC_ERR_NO_BACKING, "arena has no device memory (created with ODC_ARENA_NO_BACKING)");
   return guard.enter(a->device);
+}
+
+// What dry-run arenas have "launched" (process-wide, reset by odc_set_option("dry_run_reset", 0)).
+std::atomic<int64_t> g_dry_launches{0}, g_dry_tiles{0}, g_dry_workgroups{0};
+
+// The one place kernels are launched from. On a dry-run arena the launch is only counted: the
+// host-side validation, work-list splitting and tile tables have all run by then.
+template <class Launch>
+int launch_tiles(const odc_arena* a, void (*kernel)(const Launch), uint32_t grid, uint32_t lds_bytes, void* stream,
+                 const Launch& L) {
+  if (grid == 0 || grid > L.tt.n_tiles || L.tt.n_tiles != L.tt.tiles_per_rank * L.tt.world)
+    return fail(ODC_ERR_INVALID, "internal: launch of %u workgroups over %u tiles", grid, L.tt.n_tiles);
+  if (a->dry_run) {
+    g_dry_launches += 1;
+    g_dry_tiles += L.tt.n_tiles;
+    g_dry_workgroups += grid;
+    return ODC_OK;
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_bytes, static_cast<hipStream_t>(stream), L);
+  ODC_HIP_TRY(hipGetLastError());
+  return ODC_OK;
 }
 
 Options options_snapshot() {
@@ -738,6 +763,10 @@ const char* odc_last_error(void) { return g_err; }
 int odc_abi_version(void) { return ODC_HIP_ABI_VERSION; }
 
 int odc_set_option(const char* name, int64_t value) {
+  if (name && !strcmp(name, "dry_run_reset")) {
+    g_dry_launches = 0; g_dry_tiles = 0; g_dry_workgroups = 0;
+    return ODC_OK;
+  }
   std::lock_guard<std::mutex> lk(g_opt_mu);
   int64_t* s = option_slot(name);
   if (!s) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
@@ -747,6 +776,11 @@ int odc_set_option(const char* name, int64_t value) {
 }
 
 int odc_get_option(const char* name, int64_t* value) {
+  if (name && value) {
+    if (!strcmp(name, "dry_run_launches")) { *value = g_dry_launches.load(); return ODC_OK; }
+    if (!strcmp(name, "dry_run_tiles")) { *value = g_dry_tiles.load(); return ODC_OK; }
+    if (!strcmp(name, "dry_run_workgroups")) { *value = g_dry_workgroups.load(); return ODC_OK; }
+  }
   std::lock_guard<std::mutex> lk(g_opt_mu);
   int64_t* s = option_slot(name);
   if (!s || !value) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
@@ -760,7 +794,9 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
   *out = nullptr;
   if (world_size == 0) return fail(ODC_ERR_INVALID, "world_size must be >= 1");
   if (bytes_per_rank == 0) return fail(ODC_ERR_INVALID, "bytes_per_rank must be > 0");
-  if (flags & ~(uint32_t)ODC_ARENA_NO_BACKING) return fail(ODC_ERR_INVALID, "unknown flags 0x%x", flags);
+  if (flags & ~(uint32_t)(ODC_ARENA_NO_BACKING | ODC_ARENA_DRY_RUN))
+    return fail(ODC_ERR_INVALID, "unknown flags 0x%x", flags);
+  if (flags & ODC_ARENA_DRY_RUN) flags |= ODC_ARENA_NO_BACKING;  // a dry run never owns device memory
   odc_arena* a = new (std::nothrow) odc_arena();
   if (!a) return fail(ODC_ERR_NOMEM, "host allocation failed");
   a->world = world_size;
@@ -791,7 +827,11 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
                   (unsigned long long)bytes_per_rank, hipGetErrorString(e));
     }
     a->base = static_cast<uint8_t*>(p);
+    a->origin = a->base;
     if (a->n_cu <= 0) a->n_cu = 256;
+  } else if (flags & ODC_ARENA_DRY_RUN) {
+    a->dry_run = true;
+    a->origin = reinterpret_cast<uint8_t*>(uintptr_t(1) << 44);  // never dereferenced
   }
   a->free_[0] = a->bytes_per_rank;
   *out = a;
@@ -961,9 +1001,9 @@ int check_no_overlap(const odc_arena* a, uint32_t i, const void* dst, uint64_t d
                      uint64_t src_offset, uint64_t src_seg_bytes) {
   const uint8_t* d0 = static_cast<const uint8_t*>(dst);
   const uint8_t* d1 = d0 + dst_seg_bytes * a->world;
-  if (d1 <= a->base || d0 >= a->base + a->rank_stride * a->world) return ODC_OK;
+  if (d1 <= a->origin || d0 >= a->origin + a->rank_stride * a->world) return ODC_OK;
   for (uint32_t r = 0; r < a->world; ++r) {
-    const uint8_t* s0 = a->base + (uint64_t)r * a->rank_stride + src_offset;
+    const uint8_t* s0 = a->origin + (uint64_t)r * a->rank_stride + src_offset;
     if (d0 < s0 + src_seg_bytes && s0 < d1)
       return fail(ODC_ERR_INVALID, "item %u: dst overlaps rank %u's shard", i, r);
   }
@@ -1029,7 +1069,7 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
   uint32_t next = 0;
   while (next < n_items) {
     GatherLaunch L;
-    L.base = a->base;
+    L.base = a->origin;
     L.rank_stride = a->rank_stride;
     L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
@@ -1044,9 +1084,8 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
       ragged |= (((uintptr_t)L.item[k].dst | L.item[k].src_off | L.item[k].seg_bytes) & 15u) != 0;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles, ragged);
-    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles),
-                       static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
+    if (int rc = launch_tiles(a, gather_kernel, grid, lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles), stream, L))
+      return rc;
   }
   return ODC_OK;
 }
@@ -1078,7 +1117,7 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
   uint32_t next = 0;
   while (next < n_items) {
     CastGatherLaunch L;
-    L.base = a->base;
+    L.base = a->origin;
     L.rank_stride = a->rank_stride;
     L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = first_rank;
@@ -1090,9 +1129,8 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     if (n < 0) return n;
     if (n == 0) continue;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.cast_resident_cap, grid, L.tt.n_tiles),
-                       static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
+    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, opt.cast_resident_cap, grid, L.tt.n_tiles), stream, L))
+      return rc;
   }
   return ODC_OK;
 }
@@ -1107,7 +1145,7 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
   uint32_t next = 0;
   while (next < n_spans) {
     ClearLaunch L;
-    L.base = a->base;
+    L.base = a->origin;
     L.rank_stride = a->rank_stride;
     L.tt.order = kRanksInterleaved;  // a write-only stream runs fastest with the ranks interleaved
     L.tt.first_rank = 0;
@@ -1119,8 +1157,7 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
     if (n < 0) return n;
     if (n == 0) continue;
     const uint32_t grid = grid_for(a, opt.clear_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
+    if (int rc = launch_tiles(a, clear_kernel, grid, 0u, stream, L)) return rc;
   }
   return ODC_OK;
 }
@@ -1165,7 +1202,7 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
   uint32_t next = 0;
   while (next < n_items) {
     AccumLaunch L;
-    L.base = a->base;
+    L.base = a->origin;
     L.rank_stride = a->rank_stride;
     L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = 0;
@@ -1202,9 +1239,7 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     const uint32_t grid =
         grid_for(a, store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
     const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, cap, grid, L.tt.n_tiles),
-                       static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
+    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, cap, grid, L.tt.n_tiles), stream, L)) return rc;
   }
   return ODC_OK;
 }
@@ -1234,7 +1269,7 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
   if (!(divisor == divisor) || divisor == 0.0f) return fail(ODC_ERR_INVALID, "divisor must be a non-zero number");
   const publish_fn kernel = pick_publish(acc_dtype, out_dtype);
   if (!kernel) return fail(ODC_ERR_UNSUPPORTED, "publish from dtype %d into dtype %d is not implemented", acc_dtype, out_dtype);
-  uint8_t* region = a->base + (uint64_t)rank * a->rank_stride;
+  uint8_t* region = a->origin + (uint64_t)rank * a->rank_stride;
   for (uint32_t i = 0; i < n_items; ++i) {
     const odc_publish_item& it = items[i];
     if (it.elems == 0) continue;
@@ -1277,9 +1312,8 @@ int odc_publish(odc_arena* a, uint32_t rank, const odc_publish_item* items, uint
     if (n == 0) continue;
     // one workgroup per tile: the division sequence wants the occupancy, and the launch is short
     const uint32_t grid = grid_for(a, opt.publish_blocks_per_cu, L.tt.n_tiles);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_claim_for(a, opt.publish_resident_cap, grid, L.tt.n_tiles),
-                       static_cast<hipStream_t>(stream), L);
-    ODC_HIP_TRY(hipGetLastError());
+    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, opt.publish_resident_cap, grid, L.tt.n_tiles), stream, L))
+      return rc;
   }
   return ODC_OK;
 }
