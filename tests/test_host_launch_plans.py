@@ -50,6 +50,7 @@ def arena():
 
 
 OUTSIDE = 1 << 33  # a "device address" far from the dry-run arena's fictitious base (1 << 44)
+FAR_OUTSIDE = 1 << 50  # the same, above the arena: room for outputs of 2^46 bytes
 
 
 def test_dry_run_arena_has_no_memory_but_plans(arena):
@@ -182,7 +183,7 @@ def test_validation_errors_come_back_as_codes_and_messages(arena):
 
 def test_an_item_too_large_for_one_launch_is_refused_not_truncated(arena):
     a = arena(1, 1 << 46)
-    items = (_native.GatherItem * 1)(_native.GatherItem(OUTSIDE, 0, 1 << 46))  # 2^32 tiles
+    items = (_native.GatherItem * 1)(_native.GatherItem(FAR_OUTSIDE, 0, 1 << 46))  # 2^32 tiles
     status = a.lib.odc_gather(a.handle, items, 1, 0, None)
     assert status == _native.ODC_ERR_INVALID and "too large for one launch" in a.lib.odc_last_error().decode()
     assert a.counters() == (0, 0, 0)
@@ -198,7 +199,7 @@ def test_many_large_items_split_when_the_tile_count_would_overflow(arena):
     per_item = (1 << 29) * TILE_BYTES  # 2^29 tiles per rank, 2^30 per item
     items = (_native.GatherItem * 3)()
     for i, it in enumerate(items):
-        it.dst, it.src_offset, it.shard_bytes = OUTSIDE, i * per_item, per_item
+        it.dst, it.src_offset, it.shard_bytes = FAR_OUTSIDE, i * per_item, per_item
     _native.check(a.lib.odc_gather(a.handle, items, 3, 0, None))
     launches, tiles, _ = a.counters()
     assert (launches, tiles) == (3, 3 << 30)  # 2^30 + 2^30 would reach 2^31: one item per launch
