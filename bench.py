@@ -198,10 +198,15 @@ def measure_ceiling(torch, comm, N, iters=12):
     from odc_amd import _native
 
     lib = _native.load_ceiling()
+    # every kernel has arrays of its own: what one leaves in the 256 MB last-level cache must not
+    # be what the next one reads (a write pass over the accumulation would hand the following
+    # read-modify-write a quarter of its accumulation reads from cache)
     src = torch.empty(N, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02)
     dst = torch.empty_like(src)
     grad = torch.empty(N, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3)
     acc = torch.zeros(N, dtype=torch.float32, device="cuda")
+    read_only = torch.zeros(N, dtype=torch.float32, device="cuda")
+    write_only = torch.empty(N, dtype=torch.float32, device="cuda")
     sink = torch.zeros(4, dtype=torch.int32, device="cuda")
     stream = ctypes.c_void_p(comm.cuda_stream)
     moved = ctypes.c_uint64()
@@ -214,9 +219,9 @@ def measure_ceiling(torch, comm, N, iters=12):
         elif kind == "rmw_bf16_f32":
             rc = lib.odc_ceiling_rmw(acc.data_ptr(), grad.data_ptr(), N, wg, lds, stream, ctypes.byref(moved))
         elif kind == "read":
-            rc = lib.odc_ceiling_read(acc.data_ptr(), 4 * N, sink.data_ptr(), wg, lds, stream, ctypes.byref(moved))
+            rc = lib.odc_ceiling_read(read_only.data_ptr(), 4 * N, sink.data_ptr(), wg, lds, stream, ctypes.byref(moved))
         else:
-            rc = lib.odc_ceiling_write(acc.data_ptr(), 4 * N, wg, lds, stream, ctypes.byref(moved))
+            rc = lib.odc_ceiling_write(write_only.data_ptr(), 4 * N, wg, lds, stream, ctypes.byref(moved))
         assert rc == 0, f"ceiling kernel {kind} failed to launch"
         return moved.value
 
@@ -241,7 +246,8 @@ def measure_ceiling(torch, comm, N, iters=12):
     best = {k: max(v.values()) for k, v in table.items()}
     return {"unit": "GB/s", **best, "by_launch_shape": table,
             "note": "bare kernels of libodc_ceiling.so on flat arrays of the layer's sizes (copy 2 x 2N bytes, "
-                    "rmw 10N, read 4N, write 4N), launched alternately, HIP events per launch"}
+                    "rmw 10N, read 4N, write 4N; separate arrays per kernel), launched alternately, HIP events "
+                    "per launch"}
 
 
 def measure_launch_floor(torch, comm, group, gather, reduction, registry, W, launches=50):
