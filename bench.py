@@ -650,6 +650,7 @@ def main():
             "min_launch_ms": round(min(durations["accum"]), 5),
             "max_launch_ms": round(max(durations["accum"]), 5),
             "launches_timed": len(durations["accum"]),
+            "launch_ms_in_order": [round(x, 4) for x in durations["accum"][:2 * MICROBATCHES]],
             "practical_ceiling": ceiling,
         },
         "roofline_gather": {

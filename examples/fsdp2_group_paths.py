@@ -35,9 +35,16 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="a launch knob of the library, e.g. cast_resident_cap=4")
     args = ap.parse_args()
 
     import odc_amd as odc
+    from odc_amd import _native
+
+    for opt in args.option:
+        name, _, value = opt.partition("=")
+        _native.set_option(name, int(value))
     from odc_amd.fsdp import fsdp2
     from odc_amd.workloads import llama3_8b_layer_shapes, numel
 

@@ -12,7 +12,7 @@ scatter-accumulate launches on another, alone and together.
 
 It also compares launch shapes that matter once kernels co-reside: the gather's residency cap
 (which works by claiming LDS it never touches, so a capped gather cannot share a CU with a GEMM
-that needs its LDS) and the accumulate's persistent against its one-workgroup-per-tile launch.
+that needs its LDS) and the accumulate's one-workgroup-per-tile against its persistent launch.
 
     python examples/overlap_probe.py [--gemm 8192] [--launches 8]
 """
@@ -109,13 +109,13 @@ def main():
     report("gather, 1 persistent workgroup per CU", run_gather, {"gather_blocks_per_cu": 1})
     _native.set_option("gather_blocks_per_cu", 0)
     _native.set_option("gather_resident_cap", 4)
-    report("scatter-accumulate, 1 persistent workgroup per CU (default)", run_accum, {"accum_blocks_per_cu": 1})
+    report("scatter-accumulate, one workgroup per tile, no cap (default)", run_accum,
+           {"accum_blocks_per_cu": 0, "accum_resident_cap": 0})
     report("scatter-accumulate, one workgroup per tile, <= 4 resident per CU", run_accum,
            {"accum_blocks_per_cu": 0, "accum_resident_cap": 4})
-    report("scatter-accumulate, one workgroup per tile, no cap", run_accum,
-           {"accum_blocks_per_cu": 0, "accum_resident_cap": 0})
-    _native.set_option("accum_blocks_per_cu", 1)
-    _native.set_option("accum_resident_cap", 4)
+    report("scatter-accumulate, 1 persistent workgroup per CU", run_accum, {"accum_blocks_per_cu": 1})
+    _native.set_option("accum_blocks_per_cu", -1)
+    _native.set_option("accum_resident_cap", 0)
     torch.cuda.synchronize()
     registry.finalize()
     odc.finalize_distributed()

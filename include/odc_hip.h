@@ -211,16 +211,24 @@ int odc_publish(odc_arena* arena, uint32_t rank, const odc_publish_item* items, 
 const char* odc_last_error(void);
 int odc_abi_version(void);
 
-/* Launch-shape knobs, for measurement. "gather_blocks_per_cu", "accum_blocks_per_cu",
- * "store_blocks_per_cu", "clear_blocks_per_cu", "publish_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride loop
- * (0 = one workgroup per tile, dealt out by the hardware dispatcher); "gather_resident_cap",
- * "cast_resident_cap", "accum_resident_cap", "store_resident_cap", "publish_resident_cap": for one-workgroup-per-tile
- * launches, the most workgroups resident per CU
- * (enforced by claiming unused LDS; 0 = no cap); "rank_major" (gather; "accum_tile_order" for
- * scatter-accumulate and scatter-store: 1 = walk a rank's whole shard before the next rank, item by
- * item, 0 = interleave ranks tile by tile, 2 = rank outermost: all items' segments of rank 0, then of
- * rank 1, ...; accum_tile_order 3, its default, picks 2 for short segments and 1 otherwise);
- * "rank_stagger_bytes" (extra distance between rank regions, read when an arena is created).
+/* Launch-shape knobs, for measurement.
+ *  - "gather_blocks_per_cu", "accum_blocks_per_cu", "store_blocks_per_cu", "clear_blocks_per_cu",
+ *    "publish_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride
+ *    loop; 0 = one workgroup per tile, dealt out by the hardware dispatcher. accum_blocks_per_cu
+ *    defaults to -1: one per tile, except 1 persistent per CU when the launch's segments average
+ *    fewer than "accum_persistent_below_tiles" (128) tiles.
+ *  - "gather_resident_cap", "cast_resident_cap", "accum_resident_cap", "store_resident_cap",
+ *    "publish_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per
+ *    CU (enforced by claiming unused LDS; 0 = no cap, no claim).
+ *  - "rank_major" (gather) and "accum_tile_order" (scatter-accumulate, scatter-store): 1 = walk a
+ *    rank's whole shard before the next rank, item by item; 0 = interleave ranks tile by tile;
+ *    2 = rank outermost: all items' segments of rank 0, then of rank 1, ... accum_tile_order 3,
+ *    its default, picks 2 when segments average fewer than "accum_short_segment_tiles" (256)
+ *    tiles and 1 otherwise.
+ *  - "rank_stagger_bytes" (extra distance between rank regions), "rank_stride_align" (rank regions
+ *    start on multiples of it, default 16384 = one tile) and "alloc_align" (allocations of at
+ *    least this many bytes start on multiples of it, default 16384; smaller ones on 256): read
+ *    when an arena is created and rounded up to multiples of 256.
  * Unknown names return ODC_ERR_INVALID. Results never depend on these. */
 int odc_set_option(const char* name, int64_t value);
 int odc_get_option(const char* name, int64_t* value);

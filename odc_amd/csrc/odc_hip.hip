@@ -72,8 +72,10 @@ struct Options {
   int64_t gather_blocks_per_cu = 0;
   int64_t gather_resident_cap = 4;
   int64_t cast_resident_cap = 0;  // the read-heavy converting gather streams best uncapped
-  int64_t accum_resident_cap = 4;  // only ragged launches run one workgroup per tile
-  int64_t accum_blocks_per_cu = 1;
+  int64_t accum_resident_cap = 0;
+  int64_t accum_blocks_per_cu = -1;  // -1: by segment length (see scatter_launch)
+  int64_t accum_short_segment_tiles = 256;   // segments averaging fewer tiles: rank-outermost tile order
+  int64_t accum_persistent_below_tiles = 128;  // segments averaging fewer tiles: persistent launch shape
   int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
   int64_t store_resident_cap = 4;
   int64_t clear_blocks_per_cu = 0;
@@ -82,6 +84,8 @@ struct Options {
   int64_t rank_major = 1;        // gather: 0 = ranks interleaved, 1 = item-major, 2 = rank outermost
   int64_t accum_tile_order = 3;  // the same for scatter-accumulate / store; 3 = by segment length
   int64_t rank_stagger_bytes = 0;
+  int64_t rank_stride_align = 16384;  // rank regions start on multiples of this (read when an arena is created)
+  int64_t alloc_align = 16384;        // so do symmetric allocations at least this large
 };
 Options g_opt;
 std::mutex g_opt_mu;
@@ -90,11 +94,15 @@ int64_t* option_slot(const char* name) {
   if (!name) return nullptr;
   if (!strcmp(name, "gather_blocks_per_cu")) return &g_opt.gather_blocks_per_cu;
   if (!strcmp(name, "accum_blocks_per_cu")) return &g_opt.accum_blocks_per_cu;
+  if (!strcmp(name, "accum_short_segment_tiles")) return &g_opt.accum_short_segment_tiles;
+  if (!strcmp(name, "accum_persistent_below_tiles")) return &g_opt.accum_persistent_below_tiles;
   if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
   if (!strcmp(name, "publish_blocks_per_cu")) return &g_opt.publish_blocks_per_cu;
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
   if (!strcmp(name, "accum_tile_order")) return &g_opt.accum_tile_order;
   if (!strcmp(name, "rank_stagger_bytes")) return &g_opt.rank_stagger_bytes;
+  if (!strcmp(name, "rank_stride_align")) return &g_opt.rank_stride_align;
+  if (!strcmp(name, "alloc_align")) return &g_opt.alloc_align;
   if (!strcmp(name, "gather_resident_cap")) return &g_opt.gather_resident_cap;
   if (!strcmp(name, "cast_resident_cap")) return &g_opt.cast_resident_cap;
   if (!strcmp(name, "accum_resident_cap")) return &g_opt.accum_resident_cap;
@@ -660,6 +668,7 @@ struct odc_arena {
   int lds_per_wg_max = 64 * 1024;
   uint64_t bytes_per_rank = 0;
   uint64_t rank_stride = 0;
+  uint64_t alloc_align = 16384;
   uint8_t* base = nullptr;    // the hipMalloc (null without backing)
   uint8_t* origin = nullptr;  // what launches are planned against: base, or a fictitious address on a dry-run arena
   bool dry_run = false;
@@ -770,7 +779,8 @@ int odc_set_option(const char* name, int64_t value) {
   std::lock_guard<std::mutex> lk(g_opt_mu);
   int64_t* s = option_slot(name);
   if (!s) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
-  if (value < 0) return fail(ODC_ERR_INVALID, "option '%s' must be >= 0", name);
+  const bool may_be_auto = s == &g_opt.accum_blocks_per_cu;  // -1: chosen per launch
+  if (value < (may_be_auto ? -1 : 0)) return fail(ODC_ERR_INVALID, "option '%s' must be >= 0", name);
   *s = value;
   return ODC_OK;
 }
@@ -801,8 +811,11 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
   if (!a) return fail(ODC_ERR_NOMEM, "host allocation failed");
   a->world = world_size;
   a->flags = flags;
+  const Options opt = options_snapshot();
+  const uint64_t stride_align = std::max<uint64_t>(round_up((uint64_t)opt.rank_stride_align, kAlign), kAlign);
+  a->alloc_align = std::max<uint64_t>(round_up((uint64_t)opt.alloc_align, kAlign), kAlign);
   a->bytes_per_rank = round_up(bytes_per_rank, kAlign);
-  a->rank_stride = a->bytes_per_rank + round_up((uint64_t)options_snapshot().rank_stagger_bytes, kAlign);
+  a->rank_stride = round_up(a->bytes_per_rank + round_up((uint64_t)opt.rank_stagger_bytes, kAlign), stride_align);
   if (a->rank_stride > (~0ull) / world_size) {
     delete a;
     return fail(ODC_ERR_INVALID, "arena size overflows 64 bits");
@@ -859,11 +872,16 @@ int odc_arena_alloc(odc_arena* a, uint64_t nbytes, uint64_t* offset) {
   std::lock_guard<std::mutex> lk(a->mu);
   const uint64_t need = std::max<uint64_t>(round_up(nbytes, kAlign), kAlign);
   if (need < nbytes) return fail(ODC_ERR_INVALID, "nbytes overflows");
+  // a buffer of at least one tile starts on a tile-sized boundary, so that its tiles do not
+  // straddle 4 KiB pages; smaller ones only need the 256 bytes the vector accesses want
+  const uint64_t align = need >= a->alloc_align ? a->alloc_align : kAlign;
   for (auto it = a->free_.begin(); it != a->free_.end(); ++it) {  // first fit
-    if (it->second < need) continue;
-    const uint64_t off = it->first, sz = it->second;
+    const uint64_t blk = it->first, blk_sz = it->second;
+    const uint64_t off = round_up(blk, align);
+    if (off < blk || off - blk > blk_sz || blk_sz - (off - blk) < need) continue;
     a->free_.erase(it);
-    if (sz > need) a->free_[off + need] = sz - need;
+    if (off > blk) a->free_[blk] = off - blk;  // the gap in front stays free
+    if (blk + blk_sz > off + need) a->free_[off + need] = blk + blk_sz - (off + need);
     a->live[off] = need;
     a->in_use += need;
     a->high_water = std::max(a->high_water, off + need);
@@ -1218,17 +1236,22 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     // gradient contiguously and hops between rank regions at every segment; rank-outermost walks
     // one rank region from accumulation to accumulation (they are neighbours when registered
     // together) and hops in the gradient instead. The read-modify-write stream is the one worth
-    // keeping contiguous once segments get short (measured: +2.3 % at W=64, +5.7 % on 40 uneven
-    // parameters at W=12, -0.8 % on the layer at W=8, whose segments average 740 tiles).
+    // keeping contiguous once segments get short. Measured on the 8B layer, item-major against
+    // rank-outermost: +1.1 % at W=4, +1.6 % at W=16 (370 tiles per segment on average), -1.9 % at
+    // W=32 (185), -6 % at W=64, -10 % at W=128.
+    const uint64_t segments = (uint64_t)L.tt.n_items * a->world;
     if (opt.accum_tile_order == 3)
-      L.tt.order = (uint64_t)L.tt.n_tiles < 512ull * L.tt.n_items * a->world ? kRankOutermost : kItemMajor;
+      L.tt.order = L.tt.n_tiles < (uint64_t)opt.accum_short_segment_tiles * segments ? kRankOutermost : kItemMajor;
     else
       L.tt.order = (uint32_t)opt.accum_tile_order;
-    // The persistent shape (one workgroup per CU) streams fastest, but only while every rank's
-    // chunk of the gradient and of the accumulation starts on a 128 B line: with nothing else
-    // resident to cover for it, a workgroup whose wavefronts straddle lines, or that meets heads,
-    // tails and padding, falls behind (measured: -7 % on 16 B aligned uneven shards, against
-    // +1..3 % on line-aligned ones). Everything else runs one workgroup per tile.
+    // Launch shape. With tile-aligned rank regions and buffers, one workgroup per tile streams
+    // fastest down to segments of a few hundred tiles (measured: +1.0..2.3 % over the persistent
+    // shape at W=4..32). The persistent shape, one workgroup per CU, wins on shorter segments
+    // (+1.6 % at W=64, 92 tiles per segment; level at W=128), but only while every rank's chunk of
+    // the gradient and of the accumulation starts on a 128 B line: with nothing else resident to
+    // cover for it, a workgroup whose wavefronts straddle lines, or that meets heads, tails and
+    // padding, falls behind (measured: -7 % on 16 B aligned uneven shards). So: ragged launches
+    // and all but the shortest segments run one workgroup per tile.
     // (Measured for 16-bit gradients into fp32 accumulations; fp32 gradients, 12 B per element,
     // run 2 % faster one workgroup per tile.)
     bool ragged = !(gb == 2 && ab == 4);
@@ -1236,8 +1259,10 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
       ragged |= (L.item[k].acc_off & 127u) != 0 || ((L.item[k].seg_elems * ab) & 127u) != 0 ||
                 ((L.item[k].seg_elems * gb) & 127u) != 0 || ((uintptr_t)L.item[k].grad & 127u) != 0 ||
                 L.item[k].grad_elems != L.item[k].seg_elems * a->world;
-    const uint32_t grid =
-        grid_for(a, store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu, L.tt.n_tiles, ragged);
+    int64_t blocks_per_cu = store ? opt.store_blocks_per_cu : opt.accum_blocks_per_cu;
+    if (blocks_per_cu < 0)
+      blocks_per_cu = L.tt.n_tiles < (uint64_t)opt.accum_persistent_below_tiles * segments ? 1 : 0;
+    const uint32_t grid = grid_for(a, blocks_per_cu, L.tt.n_tiles, ragged);
     const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
     if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, cap, grid, L.tt.n_tiles), stream, L)) return rc;
   }

@@ -110,6 +110,9 @@ KNOBS = [
     {"gather_blocks_per_cu": 2, "accum_blocks_per_cu": 3, "store_blocks_per_cu": 1, "clear_blocks_per_cu": 2,
      "publish_blocks_per_cu": 1},
     {"gather_resident_cap": 1, "cast_resident_cap": 2, "accum_resident_cap": 8, "store_resident_cap": 0},
+    {"accum_blocks_per_cu": 1, "accum_resident_cap": 4},
+    {"accum_persistent_below_tiles": 1 << 30, "accum_short_segment_tiles": 0},
+    {"accum_persistent_below_tiles": 0, "accum_short_segment_tiles": 1 << 30},
 ]
 
 
@@ -122,7 +125,8 @@ def test_results_do_not_depend_on_launch_knobs(make_world, knobs):
 
     names = ["gather_blocks_per_cu", "accum_blocks_per_cu", "store_blocks_per_cu", "clear_blocks_per_cu",
              "publish_blocks_per_cu", "gather_resident_cap", "cast_resident_cap", "accum_resident_cap",
-             "store_resident_cap", "rank_major", "accum_tile_order"]
+             "store_resident_cap", "rank_major", "accum_tile_order", "accum_persistent_below_tiles",
+             "accum_short_segment_tiles"]
     saved = {n: _native.get_option(n) for n in names}
     try:
         for name, value in knobs.items():

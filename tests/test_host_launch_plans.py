@@ -94,8 +94,9 @@ def test_long_item_lists_are_split_over_launches(arena, n_items):
 def test_accumulate_launch_shapes(arena):
     W = 8
     a = arena(W)
-    # line-aligned whole shards: the persistent shape, one workgroup per CU
-    shard = 1 << 20
+    # line-aligned whole shards in SHORT segments (under 128 tiles each on average): the persistent
+    # shape, one workgroup per CU
+    shard = 1 << 18
     items = (_native.AccumItem * 2)(
         _native.AccumItem(OUTSIDE, W * shard, 0, shard), _native.AccumItem(OUTSIDE + (1 << 30), W * shard, 4 * shard, shard)
     )
@@ -110,6 +111,22 @@ def test_accumulate_launch_shapes(arena):
     items[1].grad_elems -= 5
     _native.check(a.lib.odc_scatter_accumulate(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
     assert a.counters() == (1, tiles, tiles)
+    # long segments (128 tiles and more): one workgroup per tile, unless the knob says otherwise
+    _native.set_option("dry_run_reset", 0)
+    shard = 1 << 20
+    long_items = (_native.AccumItem * 2)(
+        _native.AccumItem(OUTSIDE, W * shard, 0, shard), _native.AccumItem(OUTSIDE + (1 << 30), W * shard, 4 * shard, shard)
+    )
+    _native.check(a.lib.odc_scatter_accumulate(a.handle, long_items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+    long_tiles = 2 * W * shard // TILE_ELEMS
+    assert a.counters() == (1, long_tiles, long_tiles)
+    _native.set_option("dry_run_reset", 0)
+    _native.set_option("accum_blocks_per_cu", 2)
+    try:
+        _native.check(a.lib.odc_scatter_accumulate(a.handle, long_items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+    finally:
+        _native.set_option("accum_blocks_per_cu", -1)
+    assert a.counters() == (1, long_tiles, 2 * N_CU)
     # fewer tiles than CUs: the persistent grid shrinks to the tiles
     _native.set_option("dry_run_reset", 0)
     small = (_native.AccumItem * 1)(_native.AccumItem(OUTSIDE, W * 4096, 0, 4096))

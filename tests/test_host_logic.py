@@ -88,8 +88,9 @@ def test_arena_offsets_first_fit_and_coalescing():
 
 @pytest.mark.parametrize("seed", range(4))
 def test_arena_random_schedule_against_a_model(seed):
-    """Random allocs and frees checked against a plain first-fit model with 256 B granules: same
-    offsets, no live ranges overlapping, in-use and high-water figures, full coalescing at the end."""
+    """Random allocs and frees checked against a plain first-fit model (256 B granules; buffers of
+    a tile or more start on 16 KiB boundaries): same offsets, no live ranges overlapping, in-use
+    and high-water figures, full coalescing at the end."""
     import random
 
     rng = random.Random(seed)
@@ -100,12 +101,14 @@ def test_arena_random_schedule_against_a_model(seed):
 
     def model_alloc(n):
         need = max(256, (n + 255) // 256 * 256)
+        align = 16384 if need >= 16384 else 256
         cursor = 0
-        for off in sorted(live):
-            if off - cursor >= need:
-                return cursor, need
-            cursor = off + live[off]
-        return (cursor, need) if cap - cursor >= need else (None, need)
+        for off in sorted(live) + [cap]:  # the free blocks are the gaps between live ranges
+            start = (cursor + align - 1) // align * align
+            if off > cursor and start + need <= off:
+                return start, need
+            cursor = off + live.get(off, 0)
+        return None, need
 
     for _ in range(600):
         if live and rng.random() < 0.45:
@@ -130,6 +133,26 @@ def test_arena_random_schedule_against_a_model(seed):
         a.free(off)
     assert a.alloc(cap) == 0  # everything merged back into one block
     a.destroy()
+
+
+def test_arena_places_large_buffers_on_tile_boundaries():
+    a = utils.SymmetricArena(4, 1 << 20, backing=False)
+    assert a.info().rank_stride % 16384 == 0
+    assert a.alloc(100) == 0
+    assert a.alloc(16384) == 16384  # skips to the next tile boundary
+    assert a.alloc(300) == 256  # the gap in front is still usable
+    assert a.alloc(16383) == 32768  # rounds to 16384 bytes: aligned like the others, so not in the gap
+    assert a.alloc(15616) == 768  # under a tile: 256 B granules, fills the gap exactly
+    a.destroy()
+    _native.set_option("alloc_align", 256)
+    _native.set_option("rank_stride_align", 256)
+    try:
+        b = utils.SymmetricArena(4, 1 << 20, backing=False)
+        assert [b.alloc(n) for n in (100, 16384, 300)] == [0, 256, 16640]
+        b.destroy()
+    finally:
+        _native.set_option("alloc_align", 16384)
+        _native.set_option("rank_stride_align", 16384)
 
 
 def test_arena_is_safe_to_share_between_host_threads():
@@ -179,7 +202,7 @@ def test_sizing_run_for_the_8b_layer():
         a.alloc(numel(shape) // W * 2)  # bf16 shard
         a.alloc(numel(shape) // W * 4)  # fp32 accumulation
     need = a.info().high_water
-    assert 27_264_000 * 6 <= need <= 27_264_000 * 6 + 18 * 256
+    assert 27_264_000 * 6 <= need <= 27_264_000 * 6 + 18 * 16384  # tile-sized buffers start on 16 KiB boundaries
     a.destroy()
 
 
