@@ -52,7 +52,7 @@ def main():
     torch.cuda.set_device(0)
     shapes = [s for _, s in llama3_8b_layer_shapes()]
     N = sum(numel(s) for s in shapes)
-    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * 8 + (64 << 20))
+    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * 16 + (64 << 20))
     fsdp2.patch_fsdp2()  # creates the two services the group uses (nothing of torch is touched here)
     layer = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16,
                              reduce_dtype=torch.float32, name="layer")
@@ -93,13 +93,23 @@ def main():
     def publish_fused():
         return scatter.publish([id(layer)], out_dtype=torch.bfloat16, divisor=float(W))
 
+    unshard_row = ("unshard (fp32 shards -> bf16 parameters)", timed(lambda: unshard(False)), timed(lambda: unshard(True)), 6 * N)
+    fused_reduce = timed(lambda: layer.reduce(grads, fused=True))
+    publish_row = ("publish (acc /= W, bf16 copy; one rank)", timed(publish_reference), timed(publish_fused), 10 * N // W)
+    clear_row = ("clear (zero the fp32 accumulations of all ranks)",
+                 timed(lambda: [a.zero_() for a in scatter.get_peer_accumulations(id(layer))]),
+                 timed(scatter.clear_accumulations), 4 * N)
+    # The two-step flow lays its accumulation out like the reduce-scatter output (packed); the
+    # fused one starts every slice on a tile. A group does one or the other, so the reference flow
+    # gets a group of its own (created last: the clear above covers one accumulation only).
+    reference_layer = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16,
+                                       reduce_dtype=torch.float32, name="layer, two-step reduce")
     rows = [
-        ("unshard (fp32 shards -> bf16 parameters)", timed(lambda: unshard(False)), timed(lambda: unshard(True)), 6 * N),
-        ("reduce (bf16 gradients -> fp32 accumulations)", timed(lambda: layer.reduce(grads, fused=False)),
-         timed(lambda: layer.reduce(grads, fused=True)), 10 * N),
-        ("publish (acc /= W, bf16 copy; one rank)", timed(publish_reference), timed(publish_fused), 10 * N // W),
-        ("clear (zero the fp32 accumulations of all ranks)", timed(lambda: [a.zero_() for a in scatter.get_peer_accumulations(id(layer))]),
-         timed(scatter.clear_accumulations), 4 * N),
+        unshard_row,
+        ("reduce (bf16 gradients -> fp32 accumulations)", timed(lambda: reference_layer.reduce(grads, fused=False)),
+         fused_reduce, 10 * N),
+        publish_row,
+        clear_row,
     ]
     if args.calibrate:
         a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")

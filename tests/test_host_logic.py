@@ -375,3 +375,14 @@ def test_small_helpers(monkeypatch):
     assert utils.launch_stream_policy() == "dedicated"
     monkeypatch.delenv("ODC_COMM_STREAM")
     assert utils.launch_stream_policy() == "caller"
+
+
+def test_fsdp2_accumulation_slices_start_on_tiles():
+    """The FSDP2 group accumulation: slices of a tile (4096 elements) or more start on a multiple
+    of the tile, smaller ones are packed."""
+    from odc_amd.fsdp.fsdp2 import tile_aligned_offsets
+
+    assert tile_aligned_offsets([512, 4096, 10, 5000, 4095, 8192]) == ([0, 4096, 8192, 12288, 17288, 24576], 32768)
+    assert tile_aligned_offsets([3, 5, 7]) == ([0, 3, 8], 15)
+    assert tile_aligned_offsets([]) == ([], 0)
+    assert tile_aligned_offsets([4096, 4096]) == ([0, 4096], 8192)
