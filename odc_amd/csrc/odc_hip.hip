@@ -67,8 +67,8 @@ int fail(int code, const char* fmt, ...) {
 // ------------------------------------------------------------------------------------------------
 struct Options {
   // measured on MI355X over a Llama-3-8B layer: the gather peaks with one workgroup per tile and
-  // at most 4 of them resident per CU, the read-modify-write with 1 persistent workgroup per CU,
-  // the pure-write clear with one workgroup per tile
+  // at most 4 of them resident per CU, the read-modify-write and the pure-write clear with one
+  // workgroup per tile and no cap
   int64_t gather_blocks_per_cu = 0;
   int64_t gather_resident_cap = 4;
   int64_t cast_resident_cap = 0;  // the read-heavy converting gather streams best uncapped
@@ -744,9 +744,9 @@ Options options_snapshot() {
   return g_opt;
 }
 
-// Launches whose segments are all vector aligned run best with a few persistent workgroups per
-// CU (the knob); ragged ones (uneven shards: unaligned reads, heads and tails) hide their extra
-// latency better with one workgroup per tile, i.e. full occupancy (measured: +5..10 %).
+// blocks_per_cu > 0 asks for that many persistent workgroups per CU. Ragged launches (uneven
+// shards: unaligned reads, heads and tails) never get them: they hide their extra latency better
+// with one workgroup per tile, i.e. full occupancy (measured: +5..10 %).
 uint32_t grid_for(const odc_arena* a, int64_t blocks_per_cu, uint32_t n_tiles, bool ragged = false) {
   if (blocks_per_cu <= 0 || ragged) return n_tiles;
   const uint64_t g = (uint64_t)a->n_cu * (uint64_t)blocks_per_cu;
