@@ -113,6 +113,10 @@ KNOBS = [
     {"accum_blocks_per_cu": 1, "accum_resident_cap": 4},
     {"accum_persistent_below_tiles": 1 << 30, "accum_short_segment_tiles": 0},
     {"accum_persistent_below_tiles": 0, "accum_short_segment_tiles": 1 << 30},
+    # arena layout (read when the world is created): packed buffers and staggered, unaligned rank
+    # regions; coarse alignment
+    {"alloc_align": 256, "rank_stride_align": 256, "rank_stagger_bytes": 4352},
+    {"alloc_align": 65536, "rank_stride_align": 2 << 20},
 ]
 
 
@@ -126,7 +130,7 @@ def test_results_do_not_depend_on_launch_knobs(make_world, knobs):
     names = ["gather_blocks_per_cu", "accum_blocks_per_cu", "store_blocks_per_cu", "clear_blocks_per_cu",
              "publish_blocks_per_cu", "gather_resident_cap", "cast_resident_cap", "accum_resident_cap",
              "store_resident_cap", "rank_major", "accum_tile_order", "accum_persistent_below_tiles",
-             "accum_short_segment_tiles"]
+             "accum_short_segment_tiles", "alloc_align", "rank_stride_align", "rank_stagger_bytes"]
     saved = {n: _native.get_option(n) for n in names}
     try:
         for name, value in knobs.items():
