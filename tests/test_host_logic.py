@@ -86,22 +86,27 @@ def test_arena_offsets_first_fit_and_coalescing():
         a.alloc(1)  # use after finalize
 
 
+@pytest.mark.parametrize("big_align", [256, 4096, 16384, 65536])
 @pytest.mark.parametrize("seed", range(4))
-def test_arena_random_schedule_against_a_model(seed):
+def test_arena_random_schedule_against_a_model(seed, big_align):
     """Random allocs and frees checked against a plain first-fit model (256 B granules; buffers of
-    a tile or more start on 16 KiB boundaries): same offsets, no live ranges overlapping, in-use
+    `alloc_align` bytes or more, by default a tile, start on multiples of it): same offsets, no live ranges overlapping, in-use
     and high-water figures, full coalescing at the end."""
     import random
 
     rng = random.Random(seed)
     cap = 1 << 20
-    a = utils.SymmetricArena(3, cap, backing=False)
+    _native.set_option("alloc_align", big_align)  # read when the arena is created
+    try:
+        a = utils.SymmetricArena(3, cap, backing=False)
+    finally:
+        _native.set_option("alloc_align", 16384)
     live = {}  # offset -> rounded size
     high = 0
 
     def model_alloc(n):
         need = max(256, (n + 255) // 256 * 256)
-        align = 16384 if need >= 16384 else 256
+        align = big_align if need >= big_align else 256
         cursor = 0
         for off in sorted(live) + [cap]:  # the free blocks are the gaps between live ranges
             start = (cursor + align - 1) // align * align
