@@ -64,9 +64,12 @@ def fake_process_group():
         dist.destroy_process_group()
 
 
+@pytest.mark.parametrize("dims", [(96, 50), (192, 1100)], ids=["small", "wide"])
 @pytest.mark.parametrize("W", [4, 8])
 @pytest.mark.parametrize("mixed", [True, False])
-def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_group, W, mixed):
+def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_group, W, mixed, dims):
+    """`wide`: the weight shards exceed one tile (4096 elements), so the groups' accumulations
+    have their slices on tile boundaries, with gaps after the small ones (norms, biases)."""
     from torch.distributed.device_mesh import init_device_mesh
     from torch.distributed.fsdp import MixedPrecisionPolicy, fully_shard
 
@@ -78,7 +81,7 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
     fsdp2.patch_fsdp2()
 
     torch.manual_seed(0)
-    model = Toy().cuda()
+    model = Toy(dim=dims[0], hidden=dims[1]).cuda()
     reference = copy.deepcopy(model)
     full_params = {name: p.detach().clone() for name, p in reference.named_parameters()}
     kwargs = {"mesh": mesh}
