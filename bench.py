@@ -64,7 +64,7 @@ def parse_args():
                     help="9 per-parameter shards in one multi-tensor launch, or one flat shard")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch the timed steps eagerly instead of replaying HIP graphs")
-    ap.add_argument("--event-steps", type=int, default=16,
+    ap.add_argument("--event-steps", type=int, default=104,
                     help="eager steps with one HIP event per launch, for the per-kernel roofline figures")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the bare streaming kernels")
     ap.add_argument("--no-host-overhead", action="store_true", help="skip the host-time-per-call measurement")
@@ -647,6 +647,7 @@ def main():
             "traffic_source": traffic.get("accum", (None, None))[1],
             "algorithmic_bytes": 10 * N,
             "avg_launch_ms": round(a_ms, 5),
+            "median_launch_ms": round(statistics.median(durations["accum"]), 5),
             "min_launch_ms": round(min(durations["accum"]), 5),
             "max_launch_ms": round(max(durations["accum"]), 5),
             "launches_timed": len(durations["accum"]),
@@ -664,7 +665,9 @@ def main():
             "traffic_source": traffic.get("gather", (None, None))[1],
             "algorithmic_bytes": 4 * N,
             "avg_launch_ms": round(g_ms, 5),
+            "median_launch_ms": round(statistics.median(durations["gather"]), 5),
             "min_launch_ms": round(min(durations["gather"]), 5),
+            "launches_timed": len(durations["gather"]),
             "max_launch_ms": round(max(durations["gather"]), 5),
         },
         "clear": {"avg_launch_ms": round(c_ms, 5) if c_ms else None,
