@@ -35,6 +35,7 @@ from __future__ import annotations
 
 import logging
 import math
+import os
 from typing import List, Optional, Sequence
 
 import torch
@@ -636,6 +637,22 @@ def pre_optimizer_step(fsdp_module):
             group.update_gradients()
 
 
+def _comm_context_lazy_init(self, device):
+    """``FSDPCommContext.lazy_init`` with the all-gather and reduce-scatter streams at the default
+    priority. torch creates them at high priority so that its copy-in / copy-out kernels are not
+    delayed behind compute; the launches here gain nothing from it on MI355X (Llama example: 21.9
+    ms per microbatch with default-priority streams, 21.7-22.1 with torch's), and work queued on
+    streams of different priorities is a known hazard on this platform, which this package
+    avoids everywhere else too. ``ODC_FSDP2_STREAM_PRIORITY=torch`` keeps torch's streams."""
+    from torch.distributed.fsdp._fully_shard import _fsdp_param_group
+
+    _fsdp_param_group.FSDPCommContext._odc_original_lazy_init(self, device)
+    if os.environ.get("ODC_FSDP2_STREAM_PRIORITY", "default") != "torch":
+        self.all_gather_copy_in_stream = self.device_handle.Stream()
+        self.all_gather_stream = self.device_handle.Stream()
+        self.reduce_scatter_stream = self.device_handle.Stream()
+
+
 def patch_fsdp2(enable_hpz: bool = False) -> None:
     """Create the two services and route torch's fully_shard collectives through them
     (fsdp2.py:1105-1138). Modules sharded afterwards need ``patch_lazy_init(module)`` each."""
@@ -645,6 +662,10 @@ def patch_fsdp2(enable_hpz: bool = False) -> None:
     _enable_hpz = False
     from torch.distributed.fsdp._fully_shard import _fsdp_collectives, _fsdp_param_group
 
+    comm_context = _fsdp_param_group.FSDPCommContext
+    if not hasattr(comm_context, "_odc_original_lazy_init"):
+        comm_context._odc_original_lazy_init = comm_context.lazy_init
+        comm_context.lazy_init = _comm_context_lazy_init
     for module in (_fsdp_collectives, _fsdp_param_group):
         if not hasattr(module, "_odc_original_collectives"):
             module._odc_original_collectives = (
@@ -666,6 +687,10 @@ def unpatch_fsdp2() -> None:
         if orig is not None:
             module.foreach_all_gather, module.foreach_all_gather_copy_out, module.foreach_reduce = orig
             del module._odc_original_collectives
+    comm_context = _fsdp_param_group.FSDPCommContext
+    if hasattr(comm_context, "_odc_original_lazy_init"):
+        comm_context.lazy_init = comm_context._odc_original_lazy_init
+        del comm_context._odc_original_lazy_init
 
 
 def stop():

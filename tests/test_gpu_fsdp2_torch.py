@@ -94,6 +94,9 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
         fsdp2.patch_lazy_init(layer)
     fsdp2.patch_lazy_init(model)
     fully_shard.state(model)._lazy_init()  # moves the shards into the symmetric arena
+    comm_ctx = fully_shard.state(model)._comm_ctx
+    for s in (comm_ctx.all_gather_copy_in_stream, comm_ctx.all_gather_stream, comm_ctx.reduce_scatter_stream):
+        assert s.priority == 0  # the patch keeps every stream that carries work at the default priority
     for module in [*model.layers, model]:
         fsdp2.fill_peer_shards(module, full_params)
     breakdown = fsdp2.get_symm_buffer_memory_breakdown()
