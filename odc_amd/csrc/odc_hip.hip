@@ -890,11 +890,13 @@ int odc_arena_alloc(odc_arena* a, uint64_t nbytes, uint64_t* offset) {
     *offset = off;
     return ODC_OK;
   }
+  uint64_t largest = 0;
+  for (const auto& blk : a->free_) largest = std::max(largest, blk.second);
   return fail(ODC_ERR_NOMEM,
-              "symmetric arena exhausted: need %llu bytes per rank, %llu of %llu in use "
-              "(raise ODC_SYMMETRIC_SIZE)",
-              (unsigned long long)need, (unsigned long long)a->in_use,
-              (unsigned long long)a->bytes_per_rank);
+              "symmetric arena exhausted: need %llu bytes per rank on a %llu-byte boundary, %llu of %llu "
+              "in use, largest free block %llu (raise ODC_SYMMETRIC_SIZE)",
+              (unsigned long long)need, (unsigned long long)align, (unsigned long long)a->in_use,
+              (unsigned long long)a->bytes_per_rank, (unsigned long long)largest);
 }
 
 int odc_arena_free(odc_arena* a, uint64_t offset) {
