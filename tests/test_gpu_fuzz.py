@@ -2,6 +2,7 @@
 Every case is seeded; sizes cluster around the tile boundaries (1024 vectors = 16 KiB / 4096
 elements) where head, tail, partial-run and padding logic meet."""
 
+import os
 import random
 
 import pytest
@@ -16,11 +17,15 @@ SIZES = [0, 1, 2, 3, 5, 15, 16, 17, 63, 64, 65, 255, 1023, 4095, 4096, 4097, 819
          16399, 32768, 32771, 49153, 70001]
 
 
+# ODC_FUZZ_SEEDS=300 turns the two seeded tests below into a longer campaign
+SEEDS = range(int(os.environ.get("ODC_FUZZ_SEEDS", "12")))
+
+
 def pick_size(rng):
     return rng.choice(SIZES) if rng.random() < 0.8 else rng.randrange(0, 90_000)
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", SEEDS)
 def test_gather_random_byte_layouts(make_world, seed):
     """uint8 shards at arbitrary byte offsets inside one symmetric buffer, gathered to arbitrary
     byte offsets inside one output buffer: every alignment combination of both sides."""
@@ -63,7 +68,7 @@ PAIRS = [(torch.bfloat16, torch.float32), (torch.float32, torch.float32), (torch
          (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.bfloat16)]
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", SEEDS)
 def test_scatter_accumulate_random_slices_and_padding(make_world, seed):
     """Several gradients at arbitrary element offsets accumulated into arbitrary slices of one
     accumulation, each possibly shorter than W * shard (zero padded), twice."""
