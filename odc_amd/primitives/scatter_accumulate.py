@@ -82,11 +82,15 @@ class _AccumPlan:
     """The cached part of one scatter-accumulate call: its item array with everything but the
     gradient pointers filled in."""
 
-    __slots__ = ("items", "n", "grad_code", "acc_code", "acc_dtype", "max_numels", "tiles_exactly", "keys")
+    __slots__ = ("items", "n", "grad_code", "acc_code", "acc_dtype", "max_numels", "tiles_exactly", "keys",
+                 "layout")
 
     def __init__(self, n):
         self.items = (_native.AccumItem * n)()
         self.n = n
+
+
+_MIXED = "mixed"
 
 
 class ReductionService:
@@ -102,6 +106,11 @@ class ReductionService:
         self.lazy_clear = bool(lazy_clear)
         self._owed_zero = set()  # keys whose accumulations count as zero but hold stale bytes
         self._captured = set()  # keys ever accumulated under stream capture: always cleared by a kernel
+        # key -> what has been written into the accumulation since a kernel last zeroed all of it:
+        # None (nothing), one layout of disjoint slices, or _MIXED (anything else). A lazy clear
+        # may be folded into a store over slices only while everything outside them is still zero.
+        self._written = {}
+        self._sliced_keys = set()  # keys ever used through scatter_accumulate_slices
         self._plans = threading.local()  # per host thread: plan key -> _AccumPlan
 
     # -- registration ---------------------------------------------------------------------
@@ -134,6 +143,8 @@ class ReductionService:
         self._owed_zero.difference_update(keys)
         if not keys:
             return
+        for key in keys:
+            self._written[key] = None
         registry = SymmBufferRegistry.get_instance()
         spans = (_native.Span * len(keys))()
         for i, key in enumerate(keys):
@@ -288,6 +299,9 @@ class ReductionService:
             assert grad.is_contiguous()
             items[i].grad = grad.data_ptr()
 
+        if self._sliced_keys and not self._sliced_keys.isdisjoint(keys):
+            for key in keys:  # a whole-key write also fills what lies between a key's slices
+                self._written[key] = _MIXED
         captured = self._under_capture(keys)
         duplicates = len(set(keys)) != n
         if not duplicates and (captured or not self._owed_zero or self._owed_zero.isdisjoint(keys)):
@@ -345,12 +359,15 @@ class ReductionService:
         plan = cache.get(plan_key)
         if plan is None:
             registry = SymmBufferRegistry.get_instance()
+            if key not in self._sliced_keys:
+                self._sliced_keys.add(key)
+                self._written[key] = _MIXED  # whatever whole-key calls wrote before was not tracked
             if key not in self.accumulation_indices:
                 total = accumulation_numel
                 if total is None:
                     total = max(o + m for o, m in zip(slice_offsets, slice_numels))
                 accum_dtype = accumulation_dtype or self.accumulation_dtype or grad_dtype
-                self.register(key, (total,), grad_dtype, accum_dtype, pg)
+                self.register(key, (total,), grad_dtype, accum_dtype, pg)  # zeroes it: nothing written
             offset, acc_shape, acc_dtype = registry.offsets[self._acc_key(key)]
             plan = _AccumPlan(n)
             plan.keys = (key,)
@@ -360,14 +377,20 @@ class ReductionService:
                 plan.items[i].acc_offset = offset + off * acc_dtype.itemsize
                 plan.items[i].shard_elems = m
                 plan.max_numels.append(W * m)
-            # the store form needs the slices to tile the whole accumulation exactly once
-            end, tiles = 0, True
-            for o, m in sorted((int(o), int(m)) for o, m in zip(slice_offsets, slice_numels) if m):
-                if o != end:
-                    tiles = False
+            # The store form overwrites the slices and nothing else, so it can stand in for a
+            # clear only if the slices are disjoint and the rest of the accumulation holds zeros:
+            # either there is no rest (the slices tile the accumulation), or nothing but these
+            # very slices has been written since a kernel last zeroed all of it (self._written).
+            layout = tuple(sorted((int(o), int(m)) for o, m in zip(slice_offsets, slice_numels) if m))
+            end, disjoint, gaps = 0, True, False
+            for o, m in layout:
+                if o < end:
+                    disjoint = False
                     break
+                gaps |= o != end
                 end = o + m
-            plan.tiles_exactly = tiles and end == acc_shape[0]
+            plan.layout = layout if disjoint else None
+            plan.tiles_exactly = disjoint and not gaps and end == acc_shape[0]
             plan.grad_code = native_dtype(grad_dtype)
             plan.acc_code = native_dtype(acc_dtype)
             plan.acc_dtype = acc_dtype
@@ -380,12 +403,15 @@ class ReductionService:
             items[i].grad = grad.data_ptr()
             items[i].grad_elems = numel
         store = False
+        written = self._written.get(key, _MIXED)
         if not self._under_capture(plan.keys) and key in self._owed_zero:
-            store = plan.tiles_exactly
+            store = plan.tiles_exactly or (plan.layout is not None and written in (None, plan.layout))
             if store:
                 self._owed_zero.discard(key)
             else:
                 self._settle([key])
+                written = None
+        self._written[key] = plan.layout if plan.layout is not None and written in (None, plan.layout) else _MIXED
         self._launch(items, n, plan.grad_code, plan.acc_code, store)
         self.dispatched_tasks += 1
 

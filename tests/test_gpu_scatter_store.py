@@ -132,8 +132,10 @@ def test_lazy_clear_matches_the_oracle(make_world, seed):
 
 @pytest.mark.parametrize("seed", range(6))
 def test_slices_that_tile_the_accumulation_take_the_store_form(make_world, seed):
-    """FSDP2's group layout: the per-parameter slices cover the accumulation exactly, so the
-    first reduce of a minibatch needs no clear; slices with a gap fall back to clear + add."""
+    """FSDP2's group layout: the per-parameter slices cover the accumulation (odd seeds: all of
+    it but a gap, as the tile-aligned layout leaves them), so the first reduce of a minibatch
+    needs no clear: stale sums under the slices are overwritten, the gap still holds the zeros
+    of the registration."""
     from odc_amd import ReductionService
 
     rng = random.Random(50 + seed)
@@ -150,23 +152,97 @@ def test_slices_that_tile_the_accumulation_take_the_store_form(make_world, seed)
     total = cur
     group = make_world(W, 16 << 20)
     red = ReductionService(accumulation_dtype=acc_dtype, lazy_clear=True)
-    red.register("g", (total,), grad_dtype, acc_dtype, group)
-    red.clear_accumulations()  # lazy: "g" now owes its zeros
-    poison(red._registry_peers("g"))
+    forms = []
+    launch = red._launch
+    red._launch = lambda items, n, gc, ac, store: (forms.append(store), launch(items, n, gc, ac, store))[1]
     g = torch.Generator().manual_seed(seed)
     want = [torch.zeros(total, dtype=acc_dtype) for _ in range(W)]
     order = list(range(len(sizes)))
-    for rep in range(2):
+
+    def reduce_once():
         rng.shuffle(order)  # slice order in the call is free
         valid = [rng.choice([W * s, rng.randrange(0, W * s + 1)]) for s in sizes]
         host = [torch.randn(v, generator=g).to(grad_dtype) for v in valid]
         red.scatter_accumulate_slices("g", [host[i].cuda() for i in order], [offs[i] for i in order],
-                                      [sizes[i] for i in order], group)
+                                      [sizes[i] for i in order], group, accumulation_numel=total)
         for hg, o, s in zip(host, offs, sizes):
             padded = torch.cat([hg, torch.zeros(W * s - hg.numel(), dtype=grad_dtype)])
             oracle.scatter_accumulate([w[o : o + s] for w in want], padded)
+
+    reduce_once()  # a first minibatch: registers the accumulation (zeroed) and adds into it
+    red.clear_accumulations()  # lazy: "g" now owes its zeros
+    for w in want:
+        w.zero_()
+    for peer in red._registry_peers("g"):  # stale bytes wherever earlier launches could have left them
+        for o, s in zip(offs, sizes):
+            peer[o : o + s].view(torch.uint8).fill_(0xFF)
+    reduce_once()
+    reduce_once()
+    assert forms == [False, True, False]  # after the lazy clear: one store, then adds
     for r, acc in enumerate(red.get_peer_accumulations("g")):
         assert_bit_equal(acc, want[r], f"seed {seed}: W={W} rank {r} sizes {sizes} gap {gap}")
+
+
+def test_store_form_over_slices_needs_the_rest_of_the_accumulation_to_be_zero(make_world):
+    """Slices with gaps between them: the lazy clear is folded into a store only while nothing
+    but those slices has been written since the accumulation was last zeroed as a whole.
+    Another slice layout, or a whole-key accumulate, makes the next lazy clear a real one."""
+    from odc_amd import ReductionService
+
+    W, total = 4, 20_000
+    offs, sizes = [0, 4096, 12_288], [100, 5000, 4096]  # gaps after every slice
+    other_offs, other_sizes = [50, 9000], [200, 1000]   # another layout: overlaps the gaps of the first
+    group = make_world(W, 8 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
+    forms = []
+    launch = red._launch
+    red._launch = lambda items, n, gc, ac, store: (forms.append(store), launch(items, n, gc, ac, store))[1]
+    g = torch.Generator().manual_seed(0)
+    want = [torch.zeros(total) for _ in range(W)]
+
+    def reduce_slices(o_list, s_list):
+        host = [torch.randn(W * s, generator=g).bfloat16() for s in s_list]
+        red.scatter_accumulate_slices("g", [h.cuda() for h in host], o_list, s_list, group, accumulation_numel=total)
+        for h, o, s in zip(host, o_list, s_list):
+            oracle.scatter_accumulate([w[o : o + s] for w in want], h)
+
+    def new_minibatch():
+        red.clear_accumulations()
+        for w in want:
+            w.zero_()
+
+    def check(msg):
+        for r, acc in enumerate(red.get_peer_accumulations("g")):
+            assert_bit_equal(acc, want[r], f"{msg}: rank {r}")
+
+    reduce_slices(offs, sizes)          # registers (zeroed): read-modify-write
+    new_minibatch()
+    reduce_slices(offs, sizes)          # only this layout written so far: store
+    reduce_slices(offs, sizes)
+    assert forms == [False, True, False]
+    check("same layout")
+    new_minibatch()                     # (check() settled nothing: nothing was owed)
+    reduce_slices(other_offs, other_sizes)  # another layout while zeros are owed: real clear, then add
+    assert forms[3:] == [False]
+    check("other layout")
+    new_minibatch()
+    reduce_slices(offs, sizes)          # the other layout's data lies in this layout's gaps: real clear
+    assert forms[4:] == [False]
+    check("back to the first layout after a mixed minibatch")
+    new_minibatch()
+    reduce_slices(offs, sizes)          # that clear was a whole one and only this layout followed: store
+    assert forms[5:] == [True]
+    check("first layout again")
+    new_minibatch()
+    whole = torch.randn(W * total, generator=g).bfloat16()
+    red.scatter_accumulate("g", whole.cuda(), group)  # whole key: takes the store form itself ...
+    oracle.scatter_accumulate(want, whole)
+    assert forms[6:] == [True]
+    check("whole key")
+    new_minibatch()
+    reduce_slices(offs, sizes)          # ... and leaves data between the slices: real clear
+    assert forms[7:] == [False]
+    check("slices after a whole-key minibatch")
 
 
 def test_clear_stays_eager_under_graph_capture(make_world):
