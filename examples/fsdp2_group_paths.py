@@ -35,6 +35,9 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
+    ap.add_argument("--publish-groups", type=int, default=0, metavar="K",
+                    help="also time the publish of K layer-sized accumulations in ONE launch "
+                         "(what pre_optimizer_step does for a model's parameter groups)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="a launch knob of the library, e.g. cast_resident_cap=4")
     args = ap.parse_args()
@@ -52,7 +55,7 @@ def main():
     torch.cuda.set_device(0)
     shapes = [s for _, s in llama3_8b_layer_shapes()]
     N = sum(numel(s) for s in shapes)
-    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * 16 + (64 << 20))
+    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * (16 + 4 * args.publish_groups) + (64 << 20))
     fsdp2.patch_fsdp2()  # creates the two services the group uses (nothing of torch is touched here)
     layer = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16,
                              reduce_dtype=torch.float32, name="layer")
@@ -120,6 +123,13 @@ def main():
     print(f"{'':48s} {'reference flow':>15s} {'fused':>10s} {'fused GB/s':>11s}")
     for name, ref_ms, fused_ms, fused_bytes in rows:
         print(f"{name:48s} {ref_ms * 1e3:12.1f} us {fused_ms * 1e3:7.1f} us {fused_bytes / fused_ms / 1e6:11.0f}")
+    if args.publish_groups:
+        keys = [("extra group", k) for k in range(args.publish_groups)]
+        for key in keys:
+            scatter.register(key, (N // W,), torch.bfloat16, torch.float32, group)
+        ms = timed(lambda: scatter.publish(keys, out_dtype=torch.bfloat16, divisor=float(W)))
+        moved = 10 * (N // W) * len(keys)
+        print(f"publish of {len(keys)} such groups in one launch: {ms * 1e3:.1f} us, {moved / ms / 1e6:.0f} GB/s")
     torch.cuda.synchronize()
     fsdp2.stop()
     odc.finalize_distributed()

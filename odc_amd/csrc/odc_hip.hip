@@ -608,6 +608,7 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
       avec_t* ap = reinterpret_cast<avec_t*>(acc) + tid;
       ovec_t* op = reinterpret_cast<ovec_t*>(out) + tid;
       avec_t raw[kUnroll];
+      ovec_t cast[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) raw[u] = __builtin_nontemporal_load(ap + u * kThreads);
 #pragma unroll
@@ -623,10 +624,19 @@ __global__ __launch_bounds__(kThreads) void publish_kernel(const PublishLaunch l
             for (int k = 0; k < 4; ++k) f[k] = f[k] / launch.divisor;
           }
           raw[u] = Quad<A>::narrow(f);
-          __builtin_nontemporal_store(raw[u], ap + u * kThreads);
           Quad<A>::widen(raw[u], f);  // the copy is a cast of the ROUNDED accumulation
         }
-        if (out) __builtin_nontemporal_store(Quad<O>::narrow(f), op + u * kThreads);
+        cast[u] = Quad<O>::narrow(f);
+      }
+      // The two written streams go out one after the other, not interleaved vector by vector
+      // (measured: +6..12 %; plain instead of nontemporal stores for the copy change nothing then).
+      if (launch.divide) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(raw[u], ap + u * kThreads);
+      }
+      if (out) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(cast[u], op + u * kThreads);
       }
     } else {
       // element by element (a partial or unaligned tile), all loads before the first store
