@@ -57,23 +57,38 @@ class GatherService:
         dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)
         get_world()  # raises when there is no arena (no GPU, or init_nvshmem not called)
-        if any(not i.numel() and not o.numel() for o, i in zip(output_tensors, input_tensors)):
-            pairs = [(o, i) for o, i in zip(output_tensors, input_tensors) if i.numel() or o.numel()]
-            output_tensors, input_tensors = [o for o, _ in pairs], [i for _, i in pairs]
         if not len(input_tensors):
             return
-        registry = SymmBufferRegistry.get_instance()
         src_dtype = input_tensors[0].dtype
+        pointers, numels = [], []
         for inp in input_tensors:
             assert inp.is_cuda and inp.is_contiguous(), "shards are contiguous GPU tensors"
             assert inp.dtype == src_dtype, "one launch takes one dtype pair"
-        self._gather(
-            output_tensors,
-            [registry.symmetric_offset_of(i) for i in input_tensors],
-            [i.numel() for i in input_tensors],
-            src_dtype,
-            pg,
-        )
+            pointers.append(inp.data_ptr())
+            numels.append(inp.numel())
+        # where a shard lies in the arena follows from its address alone, so the symmetric
+        # offsets of a list of shards are looked up once per list of addresses (and host thread)
+        cache = getattr(self._plans, "offsets", None)
+        if cache is None:
+            cache = self._plans.offsets = {}
+        key = (tuple(pointers), tuple(numels))
+        known = cache.get(key)
+        if known is None:
+            registry = SymmBufferRegistry.get_instance()
+            keep = [k for k, n in enumerate(numels) if n]
+            known = cache[key] = (
+                keep if len(keep) != len(numels) else None,
+                [registry.symmetric_offset_of(input_tensors[k]) for k in keep],
+                [numels[k] for k in keep],
+            )
+        keep, offsets, kept_numels = known
+        if keep is not None:  # empty shards have empty outputs and take no part in the launch
+            for k, n in enumerate(numels):
+                assert n or not output_tensors[k].numel(), f"output {k} is not empty but its shard is"
+            output_tensors = [output_tensors[k] for k in keep]
+            if not output_tensors:
+                return
+        self._gather(output_tensors, offsets, kept_numels, src_dtype, pg)
 
     def _gather(self, outs, src_offsets, shard_numels, src_dtype, pg) -> None:
         """One launch (per 64 items): ``outs[k].view(W, -1)[r]`` = the ``shard_numels[k]`` elements

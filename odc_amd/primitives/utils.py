@@ -477,24 +477,46 @@ def get_comm_stream():
     return stream
 
 
-_launch_streams = {}  # cuda_stream handle -> torch stream with launches since the last wait
+_launch_streams = {}  # stream handle -> torch stream with launches since the last wait (None: not wrapped yet)
+
+# The two environment switches are read on every launch, so that they can be flipped at run time;
+# os.environ.get costs a microsecond per lookup (key encoding), the mapping underneath it does not.
+_ENVIRON_DATA = getattr(os.environ, "_data", None)
+_ENCODE_KEY = getattr(os.environ, "encodekey", None)
+
+
+def _fast_env_reader(name: str):
+    if isinstance(_ENVIRON_DATA, dict) and _ENCODE_KEY is not None:
+        try:
+            key, decode = _ENCODE_KEY(name), os.environ.decodevalue
+            return lambda: decode(_ENVIRON_DATA[key]) if key in _ENVIRON_DATA else None
+        except Exception:  # an os.environ without these internals: the documented way
+            pass
+    return lambda: os.environ.get(name)
+
+
+_read_policy = _fast_env_reader("ODC_COMM_STREAM")
+_read_trace = _fast_env_reader("ODC_TRACE")
 
 
 def launch_stream_policy() -> str:
     """``ODC_COMM_STREAM``: "caller" (default) launches on the caller's current stream;
     "dedicated" hops to the one comm stream and joins it on both sides, as the reference does."""
-    policy = os.environ.get("ODC_COMM_STREAM", "caller")
-    if policy not in ("caller", "dedicated"):
+    policy = _read_policy()
+    if policy is None or policy == "caller":
+        return "caller"
+    if policy != "dedicated":
         raise ValueError(f"ODC_COMM_STREAM must be 'caller' or 'dedicated', not {policy!r}")
     return policy
 
 
 def _tracing() -> bool:
-    return os.environ.get("ODC_TRACE", "0") == "1"
+    return _read_trace() == "1"
 
 
 class comm_stream_section:
-    """``with comm_stream_section(label) as stream:`` — the stream the body's launches go to.
+    """``with comm_stream_section(label) as section:`` — ``section.cuda_stream`` is the handle of
+    the stream the body's launches go to.
     With ``ODC_TRACE=1`` the section is a marker range named ``label`` (roctx through
     ``torch.cuda.nvtx``; the reference brackets the same places with NVTX,
     ``scatter_accumulate.py:307,383,736``), visible to ``rocprofv3 --marker-trace``.
@@ -508,9 +530,12 @@ class comm_stream_section:
     the same when only the gathers or only the scatter-accumulates hop, when the joins are left
     out, with 4, 8 or 16 hardware queues, and it is not a matter of stream priority (FSDP2's
     streams at default priority cost nothing).
-    ``ODC_COMM_STREAM=dedicated`` restores the hop."""
+    ``ODC_COMM_STREAM=dedicated`` restores the hop.
 
-    __slots__ = ("label", "_traced", "_current", "_comm")
+    This sits on the host path of every launch, so the default policy asks torch for the raw
+    handle of the current stream only (a stream object is built when ``sync`` needs one)."""
+
+    __slots__ = ("label", "cuda_stream", "_traced", "_current", "_comm")
 
     def __init__(self, label: str = "odc"):
         self.label = label
@@ -521,17 +546,21 @@ class comm_stream_section:
         if self._traced:
             torch.cuda.nvtx.range_push(self.label)
         try:
-            current = torch.cuda.current_stream()
             if launch_stream_policy() == "caller":
-                _launch_streams[current.cuda_stream] = current
-                return current
+                handle = torch._C._cuda_getCurrentRawStream(get_world().arena.device)
+                if handle not in _launch_streams:
+                    _launch_streams[handle] = None
+                self.cuda_stream = handle
+                return self
+            current = torch.cuda.current_stream()
             comm = get_comm_stream()
             _launch_streams[comm.cuda_stream] = comm
+            self.cuda_stream = comm.cuda_stream
             if current == comm:
-                return comm
+                return self
             comm.wait_stream(current)
             self._current, self._comm = current, comm
-            return comm
+            return self
         except BaseException:
             if self._traced:
                 torch.cuda.nvtx.range_pop()
@@ -550,7 +579,12 @@ class comm_stream_section:
 def wait_for_launches() -> None:
     """Block the host until every launch issued through ``comm_stream_section`` has finished."""
     while _launch_streams:
-        _, s = _launch_streams.popitem()
+        handle, s = _launch_streams.popitem()
+        if s is None:
+            if handle == 0:  # the default stream: ExternalStream does not wrap a null handle
+                s = torch.cuda.default_stream(get_world().arena.device)
+            else:
+                s = torch.cuda.ExternalStream(handle, device=get_world().arena.device)
         s.synchronize()
 
 
