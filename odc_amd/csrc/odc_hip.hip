@@ -253,10 +253,21 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
       u32x4 v[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) v[u] = load_stream<u32x4>(sb + (size_t)u * kThreads * 16);
+      // a whole tile that also owns its segment's head or tail (the first and last tile of a
+      // ragged segment) reads those bytes with the same round trip as its vectors
+      const bool do_head = w.head && tid < g.head;
+      const bool do_tail = w.tail && tid < g.tail;
+      const uint64_t tail_at = g.head + g.nvec * 16 + tid;
+      uint8_t head_byte = 0, tail_byte = 0;
+      if (do_head) head_byte = s[tid];
+      if (do_tail) tail_byte = s[tail_at];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], db + u * kThreads);
+      if (do_head) d[tid] = head_byte;
+      if (do_tail) d[tail_at] = tail_byte;
+    } else if (has_edges(w)) {
+      gather_edges(d, s, c.chunk, g);
     }
-    if (has_edges(w)) gather_edges(d, s, c.chunk, g);
   }
 }
 
@@ -568,14 +579,28 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
       svec_t raw[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) raw[u] = load_stream<svec_t>(sb + (size_t)u * kThreads * sizeof(svec_t));
+      // the head and the tail of the segment, when this whole tile owns them, in the same round trip
+      typedef typename Codec<S>::raw_t sraw_t;
+      typedef typename Codec<D>::raw_t draw_t;
+      const sraw_t* ss = reinterpret_cast<const sraw_t*>(s);
+      draw_t* ds = reinterpret_cast<draw_t*>(d);
+      const bool do_head = w.head && tid < g.head;
+      const bool do_tail = w.tail && tid < g.tail;
+      const uint64_t tail_at = g.head + g.nvec * 4 + tid;
+      sraw_t head_raw = 0, tail_raw = 0;
+      if (do_head) head_raw = ss[tid];
+      if (do_tail) tail_raw = ss[tail_at];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         float f[4];
         Quad<S>::widen(raw[u], f);
         __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * kThreads);
       }
+      if (do_head) ds[tid] = Codec<D>::narrow(Codec<S>::widen(head_raw));
+      if (do_tail) ds[tail_at] = Codec<D>::narrow(Codec<S>::widen(tail_raw));
+    } else if (has_edges(w)) {
+      cast_edges<S, D>(d, s, c.chunk, g);
     }
-    if (has_edges(w)) cast_edges<S, D>(d, s, c.chunk, g);
   }
 }
 
