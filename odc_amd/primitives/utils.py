@@ -514,6 +514,13 @@ def _tracing() -> bool:
     return _read_trace() == "1"
 
 
+_current_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+if _current_raw_stream is None:  # a torch without the raw accessor: ask for the stream object
+
+    def _current_raw_stream(device: int) -> int:
+        return torch.cuda.current_stream(device).cuda_stream
+
+
 class comm_stream_section:
     """``with comm_stream_section(label) as section:`` — ``section.cuda_stream`` is the handle of
     the stream the body's launches go to.
@@ -547,7 +554,7 @@ class comm_stream_section:
             torch.cuda.nvtx.range_push(self.label)
         try:
             if launch_stream_policy() == "caller":
-                handle = torch._C._cuda_getCurrentRawStream(get_world().arena.device)
+                handle = _current_raw_stream(get_world().arena.device)
                 if handle not in _launch_streams:
                     _launch_streams[handle] = None
                 self.cuda_stream = handle
