@@ -251,3 +251,72 @@ def test_llama_architecture_example_checks_bit_exactly():
         capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert "gradient shards match the unsharded model bit for bit" in proc.stdout
+
+
+@pytest.mark.parametrize("mixed", [True, False])
+def test_patched_equals_torch_fully_shard_at_world_size_one(make_world, mixed):
+    """The reference checks its FSDP2 patches by comparing a hash of the gradients with an
+    unpatched run (examples/FSDP2/utils.py:29-66, example.py). At world size 1 torch's own
+    collectives move real data on one GPU (a one-rank RCCL group), so the same comparison runs
+    here: two minibatches of three microbatches through torch's fully_shard as it is and through
+    the patched one, equal gradient shards and equal parameters after each optimizer step."""
+    import socket
+
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.fsdp import MixedPrecisionPolicy, fully_shard
+
+    from odc_amd.fsdp import fsdp2
+
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    dist.init_process_group("nccl", init_method=f"tcp://127.0.0.1:{port}", rank=0, world_size=1,
+                            device_id=torch.device("cuda", 0))
+    try:
+        mesh = init_device_mesh("cuda", (1,))
+        torch.manual_seed(3)
+        base = Toy(dim=192, hidden=300).cuda()
+        kwargs = {"mesh": mesh}
+        if mixed:
+            kwargs["mp_policy"] = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
+        g = torch.Generator().manual_seed(4)
+        minibatches = [[torch.randn(16, 32, generator=g).cuda() for _ in range(3)] for _ in range(2)]
+
+        def train(model, patched):
+            for layer in model.layers:
+                fully_shard(layer, **kwargs)
+            fully_shard(model, **kwargs)
+            if patched:
+                for layer in model.layers:
+                    fsdp2.patch_lazy_init(layer)
+                fsdp2.patch_lazy_init(model)
+            opt = torch.optim.SGD(model.parameters(), lr=0.05)
+            seen = []
+            for batches in minibatches:
+                if patched:
+                    fsdp2.pre_minibatch_start(model)
+                for x in batches:
+                    model(x).float().pow(2).mean().backward()
+                if patched:
+                    fsdp2.pre_optimizer_step(model)
+                seen.append({n: p.grad._local_tensor.detach().clone() for n, p in model.named_parameters()})
+                opt.step()
+                opt.zero_grad()
+                seen.append({n: p._local_tensor.detach().clone() for n, p in model.named_parameters()})
+            return seen
+
+        want = train(copy.deepcopy(base), patched=False)
+        make_world(1, 64 << 20)
+        fsdp2.patch_fsdp2()
+        got = train(copy.deepcopy(base), patched=True)
+        assert len(got) == len(want) == 4
+        for step, (a, b) in enumerate(zip(got, want)):
+            assert a.keys() == b.keys()
+            for name in a:
+                assert a[name].dtype == b[name].dtype and a[name].shape == b[name].shape
+                # torch.equal: a gradient that is -0 in every microbatch stays -0 under torch's
+                # `grad += new` and becomes +0 in an accumulation that starts from +0
+                assert torch.equal(a[name], b[name]), f"{'gradient' if step % 2 == 0 else 'parameter'} {name}, minibatch {step // 2}"
+    finally:
+        fsdp2.unpatch_fsdp2()
+        dist.destroy_process_group()
