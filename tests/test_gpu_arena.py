@@ -199,3 +199,25 @@ def test_tensor_ipc_handles_round_trip(make_world):
         reconstruct_tensor(handle[:10], (1,), torch.float32)
     with pytest.raises(Exception):
         get_ipc_handle(torch.zeros(4, device="cuda"))  # not in the arena
+
+
+def test_regions_and_large_buffers_start_on_tile_boundaries(make_world):
+    """Rank regions and every buffer of a tile (16 KiB) or more start on a multiple of 16 KiB of
+    the device address space, whatever alignment hipMalloc returned."""
+    from odc_amd import SymmBufferRegistry
+    from odc_amd.primitives import utils
+
+    make_world(5, 3 << 20)
+    arena = utils.get_world().arena
+    assert arena.base % 16384 == 0 and arena.rank_stride % 16384 == 0
+    registry = SymmBufferRegistry.get_instance()
+    registry.allocate_symm_buffer("small", (100,), torch.float32)
+    registry.allocate_symm_buffer("big", (5000,), torch.float32)
+    registry.allocate_symm_buffer("small2", (3,), torch.bfloat16)
+    registry.allocate_symm_buffer("big2", (8192,), torch.bfloat16)
+    for key in ("big", "big2"):
+        for peer in registry.peer_tensors[key]:
+            assert peer.data_ptr() % 16384 == 0
+    for key in ("small", "small2"):
+        for peer in registry.peer_tensors[key]:
+            assert peer.data_ptr() % 256 == 0
