@@ -56,7 +56,7 @@ class GatherService:
         pairs). Equivalent to calling ``gather_into_tensor`` pair by pair. When the outputs'
         dtype differs from the shards' (bf16/fp16/fp32 only) the conversion is fused in."""
         assert len(output_tensors) == len(input_tensors)
-        get_world()  # raises when there is no arena (no GPU, or init_nvshmem not called)
+        world = get_world()  # raises when there is no arena (no GPU, or init_nvshmem not called)
         if not len(input_tensors):
             return
         src_dtype = input_tensors[0].dtype
@@ -71,7 +71,7 @@ class GatherService:
         cache = getattr(self._plans, "offsets", None)
         if cache is None:
             cache = self._plans.offsets = {}
-        key = (tuple(pointers), tuple(numels))
+        key = (world.serial, tuple(pointers), tuple(numels))
         known = cache.get(key)
         if known is None:
             registry = SymmBufferRegistry.get_instance()
@@ -102,7 +102,7 @@ class GatherService:
         cache = getattr(self._plans, "cache", None)
         if cache is None:
             cache = self._plans.cache = {}
-        plan_key = (tuple(src_offsets), tuple(shard_numels), src_dtype, dst_dtype)
+        plan_key = (world.serial, tuple(src_offsets), tuple(shard_numels), src_dtype, dst_dtype)
         plan = cache.get(plan_key)
         if plan is None:
             plan = cache[plan_key] = _GatherPlan()

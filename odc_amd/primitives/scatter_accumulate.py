@@ -286,7 +286,7 @@ class ReductionService:
         assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
         grad_dtype = input_tensors[0].dtype
         numels = tuple(t.numel() for t in input_tensors)
-        plan_key = ("multi", tuple(keys), numels, grad_dtype,
+        plan_key = ("multi", world.serial, tuple(keys), numels, grad_dtype,
                     None if valid_numels is None else tuple(int(v) for v in valid_numels))
         cache = self._plan_cache()
         plan = cache.get(plan_key)
@@ -354,7 +354,7 @@ class ReductionService:
         W = group_size(pg)
         assert W == world.world_size, f"group size {W} != arena world size {world.world_size}"
         grad_dtype = input_tensors[0].dtype
-        plan_key = ("slices", key, tuple(slice_offsets), tuple(slice_numels), grad_dtype)
+        plan_key = ("slices", world.serial, key, tuple(slice_offsets), tuple(slice_numels), grad_dtype)
         cache = self._plan_cache()
         plan = cache.get(plan_key)
         if plan is None:

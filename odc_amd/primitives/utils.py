@@ -179,8 +179,14 @@ class SymmetricArena:
             _native.check(self._lib.odc_arena_destroy(handle))
 
 
+_world_serial = 0
+
+
 class _VirtualWorld:
     def __init__(self, arena: SymmetricArena):
+        global _world_serial
+        _world_serial += 1
+        self.serial = _world_serial  # tells one arena from the next in caches that outlive it
         self.arena = arena
         self.world_size = arena.world_size
         self.rank = 0

@@ -221,3 +221,37 @@ def test_regions_and_large_buffers_start_on_tile_boundaries(make_world):
     for key in ("small", "small2"):
         for peer in registry.peer_tensors[key]:
             assert peer.data_ptr() % 256 == 0
+
+
+def test_a_service_kept_across_arenas_does_not_reuse_stale_plans(make_world):
+    """Launch plans and shard offsets are cached inside the services; an arena created after
+    finalize_distributed() may hand out the same addresses for other offsets and another W."""
+    from helpers import assert_bit_equal, put_shards
+    from odc_amd import GatherService, ReductionService, SymmBufferRegistry
+    from odc_amd.primitives import utils
+    from oracle import odc_oracle as oracle
+
+    gather, reduction = GatherService(), ReductionService(accumulation_dtype=torch.float32)
+    g = torch.Generator().manual_seed(9)
+    S = 20_000
+    for W, pad in ((4, 0), (2, 4096), (4, 0)):
+        group = make_world(W, 4 << 20)
+        registry = SymmBufferRegistry.get_instance()
+        if pad:
+            registry.allocate_symm_buffer("pad", (pad,), torch.uint8)  # shifts every later offset
+        shards = [torch.randn(S, generator=g).bfloat16() for _ in range(W)]
+        src = put_shards(registry, "p", shards)
+        out = torch.empty(W * S, dtype=torch.bfloat16, device="cuda")
+        gather.gather_into_tensor(out, src, group)
+        assert_bit_equal(out, oracle.gather(shards), f"gather at W={W}")
+        fresh = ReductionService(accumulation_dtype=torch.float32)  # accumulations belong to one arena
+        grad = torch.randn(W * S, generator=g).bfloat16()
+        fresh.scatter_accumulate("k", grad.cuda(), group)
+        want = [torch.zeros(S) for _ in range(W)]
+        oracle.scatter_accumulate(want, grad)
+        for r, acc in enumerate(fresh.get_peer_accumulations("k")):
+            assert_bit_equal(acc, want[r], f"accumulation of rank {r} at W={W}")
+        torch.cuda.synchronize()
+        registry.finalize()
+        utils.finalize_distributed()
+    del reduction
