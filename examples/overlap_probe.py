@@ -10,9 +10,9 @@ scatter-accumulate launches on another, alone and together.
 
     hidden = (t_gemm + t_path - t_both) / t_path      1 = free, 0 = fully serialised
 
-It also compares launch shapes that matter once kernels co-reside: the gather's residency cap
+It also compares launch shapes that matter once kernels co-reside: a residency cap on the gather
 (which works by claiming LDS it never touches, so a capped gather cannot share a CU with a GEMM
-that needs its LDS) and the accumulate's one-workgroup-per-tile against its persistent launch.
+that needs its LDS) and the one-workgroup-per-tile launches against persistent ones.
 
     python examples/overlap_probe.py [--gemm 8192] [--launches 8]
 """
@@ -104,11 +104,11 @@ def main():
         hidden = (t_gemm + t_path - t_both) / t_path
         print(f"{label:62s} {t_path * 1e3:9.3f} {t_gemm * 1e3:8.3f} {t_both * 1e3:8.3f} {hidden:7.2f}")
 
-    report("gather, one workgroup per tile, <= 4 resident per CU (default)", run_gather, {"gather_resident_cap": 4})
-    report("gather, one workgroup per tile, no residency cap (no LDS claim)", run_gather, {"gather_resident_cap": 0})
+    report("gather, one 512-thread workgroup per tile (default: 4 fit a CU)", run_gather, {"gather_resident_cap": 0})
+    report("gather, one workgroup per tile, <= 2 resident per CU (LDS claim)", run_gather, {"gather_resident_cap": 2})
     report("gather, 1 persistent workgroup per CU", run_gather, {"gather_blocks_per_cu": 1})
     _native.set_option("gather_blocks_per_cu", 0)
-    _native.set_option("gather_resident_cap", 4)
+    _native.set_option("gather_resident_cap", 0)
     report("scatter-accumulate, one workgroup per tile, no cap (default)", run_accum,
            {"accum_blocks_per_cu": 0, "accum_resident_cap": 0})
     report("scatter-accumulate, one workgroup per tile, <= 4 resident per CU", run_accum,

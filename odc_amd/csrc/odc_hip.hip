@@ -10,13 +10,14 @@
 // plus the host-side symmetric arena (one hipMalloc, W rank regions, one offset valid in all).
 //
 // Launch model shared by the kernels: the work of one launch is cut into tiles of
-// kThreads * kUnroll vectors; 256-thread workgroups walk the tiles with a grid-stride loop so
-// that, at any instant, the whole chip streams one compact window of memory. Per-item
+// kThreads * kUnroll = 1024 vectors (16 KiB); workgroups of 256 threads (512 for the two
+// gathers) walk the tiles with a grid-stride loop, by default one workgroup per tile, so that,
+// at any instant, the whole chip streams one compact window of memory. Per-item
 // descriptors (<= ODC_MAX_ITEMS_PER_LAUNCH) travel BY VALUE in the kernel argument segment and
 // are read with scalar loads, so a call needs no device-side work list, no host->device copy and
 // no allocation; longer item lists are split over several launches.
 //
-// Each wavefront issues kUnroll independent 128-bit nontemporal loads per stream before the
+// Each wavefront issues its 2 or 4 independent 128-bit nontemporal loads per stream before the
 // first store: on this part the nontemporal hint on both loads and stores is worth ~15 % over
 // plain accesses for these single-touch streams. Deeper unrolling or prefetching the next tile
 // measured slower: the memory system prefers a small window to more requests in flight.
@@ -67,13 +68,21 @@ int fail(int code, const char* fmt, ...) {
 // ------------------------------------------------------------------------------------------------
 // options
 // ------------------------------------------------------------------------------------------------
+// Workgroup shape of the two gathers: 512 threads x 2 steps over the same 16 KiB tile as the
+// 256 x 4 of the other kernels. Four such workgroups fill a CU's wave slots, which is the
+// residency the copies stream best at (measured: +1.4..2.6 % over 256 x 4 with a residency cap,
+// which had to be enforced by claiming LDS; 1024 x 1 loses 20 %). The read-modify-write keeps
+// 256 x 4 (512 x 2: equal on long segments, -3 % in the persistent shape at W=64), and so does
+// the clear (512 x 2: -25 % on per-parameter spans).
+constexpr int kCopyThreads = 512;
+constexpr int kCopyUnroll = 2;
+
 struct Options {
-  // measured on MI355X over a Llama-3-8B layer: the gather peaks with one workgroup per tile and
-  // at most 4 of them resident per CU, the read-modify-write and the pure-write clear with one
-  // workgroup per tile and no cap
+  // measured on MI355X over a Llama-3-8B layer: every kernel peaks with one workgroup per tile;
+  // the scatter-store wants at most 4 of its 256-thread workgroups resident per CU
   int64_t gather_blocks_per_cu = 0;
-  int64_t gather_resident_cap = 4;
-  int64_t cast_resident_cap = 0;  // the read-heavy converting gather streams best uncapped
+  int64_t gather_resident_cap = 0;  // 512-thread workgroups: 4 per CU without a cap
+  int64_t cast_resident_cap = 0;
   int64_t accum_resident_cap = 0;
   int64_t accum_blocks_per_cu = -1;  // -1: by segment length (see scatter_launch)
   int64_t accum_short_segment_tiles = 256;   // segments averaging fewer tiles: rank-outermost tile order
@@ -206,6 +215,7 @@ __device__ __forceinline__ V load_stream(const uint8_t* p) {  // nontemporal, an
 // ---- gather -------------------------------------------------------------------------------
 // Everything of a tile that is not a run of kTileVecs whole vectors: the last partial run, the
 // head and the tail. Kept out of line so that the streaming loop stays tight.
+template <int T, int U>
 __device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t* s, uint32_t chunk, SegShape g) {
   // Every load of the tile is issued before its first store (a lone resident workgroup would
   // otherwise pay one memory round trip per step).
@@ -217,21 +227,25 @@ __device__ __attribute__((noinline)) void gather_edges(uint8_t* d, const uint8_t
   const bool do_head = w.head && tid < g.head;
   const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 16 + tid;
-  u32x4 v[kUnroll];
+  u32x4 v[U];
   uint8_t head_byte = 0, tail_byte = 0;
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u)
-    if (u * kThreads + tid < left) v[u] = load_stream<u32x4>(sb + (size_t)(u * kThreads + tid) * 16);
+  for (int u = 0; u < U; ++u)
+    if (u * T + tid < left) v[u] = load_stream<u32x4>(sb + (size_t)(u * T + tid) * 16);
   if (do_head) head_byte = s[tid];
   if (do_tail) tail_byte = s[tail_at];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u)
-    if (u * kThreads + tid < left) __builtin_nontemporal_store(v[u], db + u * kThreads + tid);
+  for (int u = 0; u < U; ++u)
+    if (u * T + tid < left) __builtin_nontemporal_store(v[u], db + u * T + tid);
   if (do_head) d[tid] = head_byte;
   if (do_tail) d[tail_at] = tail_byte;
 }
 
-__global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch launch) {
+// T threads do a tile in U steps of T vectors (T * U = kTileVecs, so the geometry is that of every
+// other kernel); the copies stream best from 512-thread workgroups, of which 4 fit a CU.
+template <int T, int U>
+__global__ __launch_bounds__(T) void gather_kernel(const GatherLaunch launch) {
+  static_assert(T * U == (int)kTileVecs, "one tile per workgroup step");
   const uint32_t tid = threadIdx.x;
   TileCursor cur;
   GatherDesc it = {};
@@ -250,9 +264,9 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
     if (is_whole(w)) {
       const uint8_t* sb = s + g.head + (w.v0 + tid) * 16;
       u32x4* db = reinterpret_cast<u32x4*>(d + g.head) + w.v0 + tid;
-      u32x4 v[kUnroll];
+      u32x4 v[U];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) v[u] = load_stream<u32x4>(sb + (size_t)u * kThreads * 16);
+      for (int u = 0; u < U; ++u) v[u] = load_stream<u32x4>(sb + (size_t)u * T * 16);
       // a whole tile that also owns its segment's head or tail (the first and last tile of a
       // ragged segment) reads those bytes with the same round trip as its vectors
       const bool do_head = w.head && tid < g.head;
@@ -262,11 +276,11 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const GatherLaunch lau
       if (do_head) head_byte = s[tid];
       if (do_tail) tail_byte = s[tail_at];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], db + u * kThreads);
+      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], db + u * T);
       if (do_head) d[tid] = head_byte;
       if (do_tail) d[tail_at] = tail_byte;
     } else if (has_edges(w)) {
-      gather_edges(d, s, c.chunk, g);
+      gather_edges<T, U>(d, s, c.chunk, g);
     }
   }
 }
@@ -511,7 +525,7 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
 // ---- gather with cast ---------------------------------------------------------------------
 // dst[r*S + i] = narrow_D(widen_S(region_r[off + i])): the gather of shards kept in one dtype
 // (fp32 master copies) into a full parameter of another (bf16), in one pass.
-template <class S, class D>
+template <class S, class D, int T, int U>
 __device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* s, uint32_t chunk, SegShape g) {
   typedef typename Quad<S>::vec_t svec_t;
   typedef typename Quad<D>::vec_t dvec_t;
@@ -530,18 +544,18 @@ __device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* 
   const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 4 + tid;
   // every load of the tile before its first store
-  svec_t raw[kUnroll];
+  svec_t raw[U];
   sraw_t head_raw = 0, tail_raw = 0;
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const uint32_t q = u * kThreads + tid;
+  for (int u = 0; u < U; ++u) {
+    const uint32_t q = u * T + tid;
     if (q < left) raw[u] = load_stream<svec_t>(sb + (size_t)q * sizeof(svec_t));
   }
   if (do_head) head_raw = ss[tid];
   if (do_tail) tail_raw = ss[tail_at];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const uint32_t q = u * kThreads + tid;
+  for (int u = 0; u < U; ++u) {
+    const uint32_t q = u * T + tid;
     if (q < left) {
       float f[4];
       Quad<S>::widen(raw[u], f);
@@ -552,8 +566,9 @@ __device__ __attribute__((noinline)) void cast_edges(uint8_t* d, const uint8_t* 
   if (do_tail) ds[tail_at] = Codec<D>::narrow(Codec<S>::widen(tail_raw));
 }
 
-template <class S, class D>
-__global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherLaunch launch) {
+template <class S, class D, int T, int U>
+__global__ __launch_bounds__(T) void cast_gather_kernel(const CastGatherLaunch launch) {
+  static_assert(T * U == (int)kTileVecs, "one tile per workgroup step");
   typedef typename Quad<S>::vec_t svec_t;
   typedef typename Quad<D>::vec_t dvec_t;
   constexpr uint32_t kSB = Codec<S>::kBytes, kDB = Codec<D>::kBytes;
@@ -576,9 +591,9 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
       const uint64_t e0 = g.head + w.v0 * 4;
       const uint8_t* sb = s + e0 * kSB + (size_t)tid * sizeof(svec_t);
       dvec_t* dp = reinterpret_cast<dvec_t*>(d + e0 * kDB) + tid;
-      svec_t raw[kUnroll];
+      svec_t raw[U];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) raw[u] = load_stream<svec_t>(sb + (size_t)u * kThreads * sizeof(svec_t));
+      for (int u = 0; u < U; ++u) raw[u] = load_stream<svec_t>(sb + (size_t)u * T * sizeof(svec_t));
       // the head and the tail of the segment, when this whole tile owns them, in the same round trip
       typedef typename Codec<S>::raw_t sraw_t;
       typedef typename Codec<D>::raw_t draw_t;
@@ -591,15 +606,15 @@ __global__ __launch_bounds__(kThreads) void cast_gather_kernel(const CastGatherL
       if (do_head) head_raw = ss[tid];
       if (do_tail) tail_raw = ss[tail_at];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
+      for (int u = 0; u < U; ++u) {
         float f[4];
         Quad<S>::widen(raw[u], f);
-        __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * kThreads);
+        __builtin_nontemporal_store(Quad<D>::narrow(f), dp + u * T);
       }
       if (do_head) ds[tid] = Codec<D>::narrow(Codec<S>::widen(head_raw));
       if (do_tail) ds[tail_at] = Codec<D>::narrow(Codec<S>::widen(tail_raw));
     } else if (has_edges(w)) {
-      cast_edges<S, D>(d, s, c.chunk, g);
+      cast_edges<S, D, T, U>(d, s, c.chunk, g);
     }
   }
 }
@@ -763,7 +778,7 @@ std::atomic<int64_t> g_dry_launches{0}, g_dry_tiles{0}, g_dry_workgroups{0};
 // host-side validation, work-list splitting and tile tables have all run by then.
 template <class Launch>
 int launch_tiles(const odc_arena* a, void (*kernel)(const Launch), uint32_t grid, uint32_t lds_bytes, void* stream,
-                 const Launch& L) {
+                 const Launch& L, uint32_t threads = kThreads) {
   if (grid == 0 || grid > L.tt.n_tiles || L.tt.n_tiles != L.tt.tiles_per_rank * L.tt.world)
     return fail(ODC_ERR_INVALID, "internal: launch of %u workgroups over %u tiles", grid, L.tt.n_tiles);
   if (a->dry_run) {
@@ -772,7 +787,7 @@ int launch_tiles(const odc_arena* a, void (*kernel)(const Launch), uint32_t grid
     g_dry_workgroups += grid;
     return ODC_OK;
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_bytes, static_cast<hipStream_t>(stream), L);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds_bytes, static_cast<hipStream_t>(stream), L);
   ODC_HIP_TRY(hipGetLastError());
   return ODC_OK;
 }
@@ -1096,7 +1111,7 @@ accum_fn pick_accum(int g, int a, bool store) {  // (gradient dtype, accumulatio
 }
 
 cast_gather_fn pick_cast_gather(int s, int d) {  // (shard dtype, output dtype)
-#define X(E1, T1, E2, T2) if (s == E1 && d == E2) return cast_gather_kernel<T1, T2>;
+#define X(E1, T1, E2, T2) if (s == E1 && d == E2) return cast_gather_kernel<T1, T2, kCopyThreads, kCopyUnroll>;
   ODC_FOR_EACH_DTYPE_PAIR(X)
 #undef X
   return nullptr;
@@ -1146,7 +1161,8 @@ int odc_gather(odc_arena* a, const odc_gather_item* items, uint32_t n_items, uin
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
       ragged |= (((uintptr_t)L.item[k].dst | L.item[k].src_off | L.item[k].seg_bytes) & 15u) != 0;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles, ragged);
-    if (int rc = launch_tiles(a, gather_kernel, grid, lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles), stream, L))
+    if (int rc = launch_tiles(a, gather_kernel<kCopyThreads, kCopyUnroll>, grid,
+                              lds_claim_for(a, opt.gather_resident_cap, grid, L.tt.n_tiles), stream, L, kCopyThreads))
       return rc;
   }
   return ODC_OK;
@@ -1191,7 +1207,8 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
     if (n < 0) return n;
     if (n == 0) continue;
     const uint32_t grid = grid_for(a, opt.gather_blocks_per_cu, L.tt.n_tiles);
-    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, opt.cast_resident_cap, grid, L.tt.n_tiles), stream, L))
+    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, opt.cast_resident_cap, grid, L.tt.n_tiles), stream, L,
+                              kCopyThreads))
       return rc;
   }
   return ODC_OK;
