@@ -194,7 +194,7 @@ def load_traffic(args, W):
 def measure_ceiling(torch, comm, N, iters=12):
     """Bare streaming kernels over flat arrays of the layer's sizes, launched alternately (copy,
     read-modify-write, read, write: every launch meets cold caches, as the real steps do) with
-    one HIP event after each. Three launch shapes each; the best average is the ceiling."""
+    one HIP event after each. Four launch shapes each; the best average is the ceiling."""
     from odc_amd import _native
 
     lib = _native.load_ceiling()
@@ -210,8 +210,9 @@ def measure_ceiling(torch, comm, N, iters=12):
     sink = torch.zeros(4, dtype=torch.int32, device="cuda")
     stream = ctypes.c_void_p(comm.cuda_stream)
     moved = ctypes.c_uint64()
-    shapes = {"one workgroup per tile": (0, 0), "one per tile, 4 resident per CU": (0, 40960),
-              "1 persistent workgroup per CU": (1, 0)}
+    # (persistent workgroups per CU or 0, unused LDS claimed per workgroup, threads per workgroup)
+    shapes = {"one workgroup per tile": (0, 0, 256), "one per tile, 4 resident per CU": (0, 40960, 256),
+              "1 persistent workgroup per CU": (1, 0, 256), "one 512-thread workgroup per tile": (0, 0, 512)}
 
     def launch(kind, wg, lds):
         if kind == "copy":
@@ -228,7 +229,8 @@ def measure_ceiling(torch, comm, N, iters=12):
     kinds = ("copy", "rmw_bf16_f32", "read", "write")
     table = {k: {} for k in kinds}
     with torch.cuda.stream(comm):
-        for label, (wg, lds) in shapes.items():
+        for label, (wg, lds, threads) in shapes.items():
+            assert lib.odc_ceiling_set_threads(threads) == 0
             marks, nbytes = [], {}
             for it in range(iters + 2):
                 for kind in kinds:

@@ -179,7 +179,9 @@ def load_ceiling() -> ctypes.CDLL:
     lib.odc_ceiling_write.argtypes = [vp, u64, ci, u32, vp, P(u64)]
     lib.odc_ceiling_copy.argtypes = [vp, vp, u64, ci, u32, vp, P(u64)]
     lib.odc_ceiling_rmw.argtypes = [vp, vp, u64, ci, u32, vp, P(u64)]
-    for name in ("odc_ceiling_read", "odc_ceiling_write", "odc_ceiling_copy", "odc_ceiling_rmw"):
+    lib.odc_ceiling_set_threads.argtypes = [ci]
+    for name in ("odc_ceiling_read", "odc_ceiling_write", "odc_ceiling_copy", "odc_ceiling_rmw",
+                 "odc_ceiling_set_threads"):
         getattr(lib, name).restype = ci
     return lib
 

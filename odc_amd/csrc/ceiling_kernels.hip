@@ -8,8 +8,9 @@
 //   copy   : dst[i] = src[i]                                          (read 1 + write 1 per byte)
 //   rmw    : acc[i] += widen(grad[i]), bf16 -> fp32                   (10 B per element)
 //
-// Same shape as the product kernels: 256-thread workgroups, 4 independent 128-bit nontemporal
-// loads per stream per lane before the first store, one 16 KiB tile per step, grid-stride.
+// Same shapes as the product kernels: 256-thread workgroups with 4, or 512-thread workgroups
+// with 2 (odc_ceiling_set_threads), independent 128-bit nontemporal loads per stream per lane
+// before the first store, one 16 KiB tile per step, grid-stride.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -19,10 +20,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
-constexpr uint64_t kTileVecs = kThreads * kUnroll;
+constexpr uint64_t kTileVecs = 1024;  // 16 KiB of the 16-byte stream per tile
+int g_threads = 256;                  // workgroup size of the next launches: 256 (x4) or 512 (x2)
 
+template <int kThreads, int kUnroll>
 __global__ __launch_bounds__(kThreads) void read_kernel(const u32x4* src, uint64_t n_tiles, uint32_t* sink) {
   u32x4 sum = {0u, 0u, 0u, 0u};
   for (uint64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
@@ -36,6 +37,7 @@ __global__ __launch_bounds__(kThreads) void read_kernel(const u32x4* src, uint64
   if ((sum.x ^ sum.y ^ sum.z ^ sum.w) == 0x9e3779b9u) *sink = 1;  // keeps the loads alive
 }
 
+template <int kThreads, int kUnroll>
 __global__ __launch_bounds__(kThreads) void write_kernel(u32x4* dst, uint64_t n_tiles) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
   for (uint64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
@@ -45,6 +47,7 @@ __global__ __launch_bounds__(kThreads) void write_kernel(u32x4* dst, uint64_t n_
   }
 }
 
+template <int kThreads, int kUnroll>
 __global__ __launch_bounds__(kThreads) void copy_kernel(u32x4* dst, const u32x4* src, uint64_t n_tiles) {
   for (uint64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
     const u32x4* s = src + t * kTileVecs + threadIdx.x;
@@ -57,6 +60,7 @@ __global__ __launch_bounds__(kThreads) void copy_kernel(u32x4* dst, const u32x4*
   }
 }
 
+template <int kThreads, int kUnroll>
 __global__ __launch_bounds__(kThreads) void rmw_kernel(f32x4* acc, const u32x2* grad, uint64_t n_tiles) {
   for (uint64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
     f32x4* a = acc + t * kTileVecs + threadIdx.x;
@@ -95,6 +99,14 @@ int finish() { return hipGetLastError() == hipSuccess ? 0 : -1; }
 
 extern "C" {
 
+// Workgroup size of the launches that follow: 256 threads (4 loads per lane) or 512 (2 per lane).
+// Returns 0, or -1 for any other value.
+int odc_ceiling_set_threads(int threads) {
+  if (threads != 256 && threads != 512) return -1;
+  g_threads = threads;
+  return 0;
+}
+
 // Each call launches one kernel over whole tiles only: the sizes are rounded DOWN to a multiple
 // of a tile (16 KiB of the 16-byte stream; 4096 elements for rmw) and the number of bytes the
 // launch really moves is returned through *moved. lds_bytes is dynamic LDS the kernel never
@@ -105,9 +117,14 @@ int odc_ceiling_read(const void* src, uint64_t nbytes, void* sink, int workgroup
   const uint64_t n_tiles = nbytes / (kTileVecs * 16);
   if (moved) *moved = n_tiles * kTileVecs * 16;
   if (!n_tiles) return 0;
-  hipLaunchKernelGGL(read_kernel, dim3(grid_for(n_tiles, workgroups_per_cu)), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), static_cast<const u32x4*>(src), n_tiles,
-                     static_cast<uint32_t*>(sink));
+  const dim3 grid(grid_for(n_tiles, workgroups_per_cu));
+  hipStream_t q = static_cast<hipStream_t>(stream);
+  if (g_threads == 512)
+    hipLaunchKernelGGL((read_kernel<512, 2>), grid, dim3(512), lds_bytes, q, static_cast<const u32x4*>(src), n_tiles,
+                       static_cast<uint32_t*>(sink));
+  else
+    hipLaunchKernelGGL((read_kernel<256, 4>), grid, dim3(256), lds_bytes, q, static_cast<const u32x4*>(src), n_tiles,
+                       static_cast<uint32_t*>(sink));
   return finish();
 }
 
@@ -116,8 +133,12 @@ int odc_ceiling_write(void* dst, uint64_t nbytes, int workgroups_per_cu, uint32_
   const uint64_t n_tiles = nbytes / (kTileVecs * 16);
   if (moved) *moved = n_tiles * kTileVecs * 16;
   if (!n_tiles) return 0;
-  hipLaunchKernelGGL(write_kernel, dim3(grid_for(n_tiles, workgroups_per_cu)), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst), n_tiles);
+  const dim3 grid(grid_for(n_tiles, workgroups_per_cu));
+  hipStream_t q = static_cast<hipStream_t>(stream);
+  if (g_threads == 512)
+    hipLaunchKernelGGL((write_kernel<512, 2>), grid, dim3(512), lds_bytes, q, static_cast<u32x4*>(dst), n_tiles);
+  else
+    hipLaunchKernelGGL((write_kernel<256, 4>), grid, dim3(256), lds_bytes, q, static_cast<u32x4*>(dst), n_tiles);
   return finish();
 }
 
@@ -126,9 +147,14 @@ int odc_ceiling_copy(void* dst, const void* src, uint64_t nbytes, int workgroups
   const uint64_t n_tiles = nbytes / (kTileVecs * 16);
   if (moved) *moved = 2 * n_tiles * kTileVecs * 16;
   if (!n_tiles) return 0;
-  hipLaunchKernelGGL(copy_kernel, dim3(grid_for(n_tiles, workgroups_per_cu)), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst), static_cast<const u32x4*>(src),
-                     n_tiles);
+  const dim3 grid(grid_for(n_tiles, workgroups_per_cu));
+  hipStream_t q = static_cast<hipStream_t>(stream);
+  if (g_threads == 512)
+    hipLaunchKernelGGL((copy_kernel<512, 2>), grid, dim3(512), lds_bytes, q, static_cast<u32x4*>(dst),
+                       static_cast<const u32x4*>(src), n_tiles);
+  else
+    hipLaunchKernelGGL((copy_kernel<256, 4>), grid, dim3(256), lds_bytes, q, static_cast<u32x4*>(dst),
+                       static_cast<const u32x4*>(src), n_tiles);
   return finish();
 }
 
@@ -137,9 +163,14 @@ int odc_ceiling_rmw(void* acc_f32, const void* grad_bf16, uint64_t n_elems, int 
   const uint64_t n_tiles = n_elems / (kTileVecs * 4);
   if (moved) *moved = 10 * n_tiles * kTileVecs * 4;
   if (!n_tiles) return 0;
-  hipLaunchKernelGGL(rmw_kernel, dim3(grid_for(n_tiles, workgroups_per_cu)), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), static_cast<f32x4*>(acc_f32),
-                     static_cast<const u32x2*>(grad_bf16), n_tiles);
+  const dim3 grid(grid_for(n_tiles, workgroups_per_cu));
+  hipStream_t q = static_cast<hipStream_t>(stream);
+  if (g_threads == 512)
+    hipLaunchKernelGGL((rmw_kernel<512, 2>), grid, dim3(512), lds_bytes, q, static_cast<f32x4*>(acc_f32),
+                       static_cast<const u32x2*>(grad_bf16), n_tiles);
+  else
+    hipLaunchKernelGGL((rmw_kernel<256, 4>), grid, dim3(256), lds_bytes, q, static_cast<f32x4*>(acc_f32),
+                       static_cast<const u32x2*>(grad_bf16), n_tiles);
   return finish();
 }
 

@@ -640,10 +640,12 @@ def pre_optimizer_step(fsdp_module):
 def _comm_context_lazy_init(self, device):
     """``FSDPCommContext.lazy_init`` with the all-gather and reduce-scatter streams at the default
     priority. torch creates them at high priority so that its copy-in / copy-out kernels are not
-    delayed behind compute; the launches here gain nothing from it on MI355X (Llama example: 21.9
-    ms per microbatch with default-priority streams, 21.7-22.1 with torch's), and work queued on
-    streams of different priorities is a known hazard on this platform, which this package
-    avoids everywhere else too. ``ODC_FSDP2_STREAM_PRIORITY=torch`` keeps torch's streams."""
+    delayed behind compute; the launches here gain nothing from it on MI355X (Llama example: 21.8
+    ms per microbatch with default-priority streams, 21.7 with torch's), work queued on streams
+    of different priorities is a known hazard on this platform, and it is costly: with the
+    launches on the reference's dedicated comm stream (default priority) next to torch's
+    high-priority streams the same microbatch takes 28.2 ms, with all streams at the default
+    priority 21.6. ``ODC_FSDP2_STREAM_PRIORITY=torch`` keeps torch's streams."""
     from torch.distributed.fsdp._fully_shard import _fsdp_param_group
 
     _fsdp_param_group.FSDPCommContext._odc_original_lazy_init(self, device)
