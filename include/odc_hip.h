@@ -223,7 +223,7 @@ int odc_abi_version(void);
  *    fewer than "accum_persistent_below_tiles" (128) tiles.
  *  - "gather_resident_cap", "cast_resident_cap", "accum_resident_cap", "store_resident_cap",
  *    "publish_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per
- *    CU (enforced by claiming unused LDS; 0 = no cap, no claim).
+ *    CU (enforced by claiming unused LDS; 0 = no cap, no claim; all default to 0).
  *  - "rank_major" (gather) and "accum_tile_order" (scatter-accumulate, scatter-store): 1 = walk a
  *    rank's whole shard before the next rank, item by item; 0 = interleave ranks tile by tile;
  *    2 = rank outermost: all items' segments of rank 0, then of rank 1, ... accum_tile_order 3,

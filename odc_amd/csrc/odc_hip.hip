@@ -11,7 +11,7 @@
 //
 // Launch model shared by the kernels: the work of one launch is cut into tiles of
 // kThreads * kUnroll = 1024 vectors (16 KiB); workgroups of 256 threads (512 for the two
-// gathers) walk the tiles with a grid-stride loop, by default one workgroup per tile, so that,
+// gathers and the scatter-store) walk the tiles with a grid-stride loop, by default one workgroup per tile, so that,
 // at any instant, the whole chip streams one compact window of memory. Per-item
 // descriptors (<= ODC_MAX_ITEMS_PER_LAUNCH) travel BY VALUE in the kernel argument segment and
 // are read with scalar loads, so a call needs no device-side work list, no host->device copy and
@@ -68,18 +68,22 @@ int fail(int code, const char* fmt, ...) {
 // ------------------------------------------------------------------------------------------------
 // options
 // ------------------------------------------------------------------------------------------------
-// Workgroup shape of the two gathers: 512 threads x 2 steps over the same 16 KiB tile as the
-// 256 x 4 of the other kernels. Four such workgroups fill a CU's wave slots, which is the
-// residency the copies stream best at (measured: +1.4..2.6 % over 256 x 4 with a residency cap,
-// which had to be enforced by claiming LDS; 1024 x 1 loses 20 %). The read-modify-write keeps
-// 256 x 4 (512 x 2: equal on long segments, -3 % in the persistent shape at W=64), and so does
-// the clear (512 x 2: -25 % on per-parameter spans).
+// Workgroup shape of the two gathers and of the scatter-store (the kernels that read one stream
+// and write one): 512 threads x 2 steps over the same 16 KiB tile as the 256 x 4 of the other
+// kernels. Four such workgroups fill a CU's wave slots, which is the residency these kernels
+// stream best at (measured: gathers +1.4..2.6 % over 256 x 4 with a residency cap of 4, which
+// had to be enforced by claiming LDS; scatter-store level with it on per-parameter shards at W=8
+// and +2..3 % on flat shards and at W=64; 256 x 4 without a cap loses 6..8 %; 1024 x 1 loses
+// 20 %). The read-modify-write keeps 256 x 4 (512 x 2: equal on long segments, -3 % in the
+// persistent shape at W=64), and so does the clear (512 x 2: -25 % on per-parameter spans).
 constexpr int kCopyThreads = 512;
 constexpr int kCopyUnroll = 2;
+constexpr int kStoreThreads = 512;
+constexpr int kStoreUnroll = 2;
 
 struct Options {
-  // measured on MI355X over a Llama-3-8B layer: every kernel peaks with one workgroup per tile;
-  // the scatter-store wants at most 4 of its 256-thread workgroups resident per CU
+  // measured on MI355X over a Llama-3-8B layer: every kernel peaks with one workgroup per tile
+  // and no residency cap
   int64_t gather_blocks_per_cu = 0;
   int64_t gather_resident_cap = 0;  // 512-thread workgroups: 4 per CU without a cap
   int64_t cast_resident_cap = 0;
@@ -88,7 +92,7 @@ struct Options {
   int64_t accum_short_segment_tiles = 256;   // segments averaging fewer tiles: rank-outermost tile order
   int64_t accum_persistent_below_tiles = 128;  // segments averaging fewer tiles: persistent launch shape
   int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
-  int64_t store_resident_cap = 4;
+  int64_t store_resident_cap = 0;  // 512-thread workgroups, like the gathers
   int64_t clear_blocks_per_cu = 0;
   int64_t publish_blocks_per_cu = 0;
   int64_t publish_resident_cap = 0;
@@ -409,7 +413,7 @@ template <> struct Quad<f16_tag> {
 // holding -0 becomes +0, as F.pad followed by add_ leaves it). Two phases, every load of the tile
 // before its first store: a lone resident workgroup would otherwise pay one memory round trip
 // per quad.
-template <class G, class A, bool kStore>
+template <class G, class A, bool kStore, int T, int U>
 __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_t* grad, uint64_t g_seg,
                                                       uint64_t grad_elems, uint32_t chunk, SegShape g,
                                                       bool body) {
@@ -429,12 +433,12 @@ __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_
   const bool do_tail = w.tail && tid < g.tail;
   const uint64_t tail_at = g.head + g.nvec * 4 + tid;
 
-  float gf[kUnroll][4];
-  avec_t araw[kUnroll];
+  float gf[U][4];
+  avec_t araw[U];
   float head_g = 0.0f, head_a = 0.0f, tail_g = 0.0f, tail_a = 0.0f;
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const uint32_t q = u * kThreads + tid;
+  for (int u = 0; u < U; ++u) {
+    const uint32_t q = u * T + tid;
 #pragma unroll
     for (int k = 0; k < 4; ++k) gf[u][k] = 0.0f;
     if (q < left) {
@@ -459,8 +463,8 @@ __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_
   }
 
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const uint32_t q = u * kThreads + tid;
+  for (int u = 0; u < U; ++u) {
+    const uint32_t q = u * T + tid;
     if (q < left) {
       float af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
       if constexpr (!kStore) Quad<A>::widen(araw[u], af);
@@ -473,8 +477,9 @@ __device__ __attribute__((noinline)) void accum_edges(uint8_t* acc, const uint8_
   if (do_tail) as[tail_at] = Codec<A>::narrow(tail_a + tail_g);
 }
 
-template <class G, class A, bool kStore>
-__global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launch) {
+template <class G, class A, bool kStore, int T, int U>
+__global__ __launch_bounds__(T) void accum_kernel(const AccumLaunch launch) {
+  static_assert(T * U == (int)kTileVecs, "one tile per workgroup step");
   typedef typename Quad<G>::vec_t gvec_t;
   typedef typename Quad<A>::vec_t avec_t;
   constexpr uint32_t kAB = Codec<A>::kBytes, kGB = Codec<G>::kBytes;
@@ -499,26 +504,26 @@ __global__ __launch_bounds__(kThreads) void accum_kernel(const AccumLaunch launc
     if (whole) {
       const uint8_t* gb = it.grad + (g_seg + e0) * kGB + (size_t)tid * sizeof(gvec_t);
       avec_t* ap = reinterpret_cast<avec_t*>(acc + e0 * kAB) + tid;
-      gvec_t graw[kUnroll];
-      avec_t araw[kUnroll];
+      gvec_t graw[U];
+      avec_t araw[U];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) graw[u] = load_stream<gvec_t>(gb + (size_t)u * kThreads * sizeof(gvec_t));
+      for (int u = 0; u < U; ++u) graw[u] = load_stream<gvec_t>(gb + (size_t)u * T * sizeof(gvec_t));
       if constexpr (!kStore) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) araw[u] = __builtin_nontemporal_load(ap + u * kThreads);
+        for (int u = 0; u < U; ++u) araw[u] = __builtin_nontemporal_load(ap + u * T);
       }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
+      for (int u = 0; u < U; ++u) {
         float gf[4], af[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         Quad<G>::widen(graw[u], gf);
         if constexpr (!kStore) Quad<A>::widen(araw[u], af);
 #pragma unroll
         for (int k = 0; k < 4; ++k) af[k] = af[k] + gf[k];
-        __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * kThreads);
+        __builtin_nontemporal_store(Quad<A>::narrow(af), ap + u * T);
       }
     }
     if (!whole ? (w.nv != 0 || w.head || w.tail) : (w.head || w.tail))
-      accum_edges<G, A, kStore>(acc, it.grad, g_seg, it.grad_elems, c.chunk, g, !whole);
+      accum_edges<G, A, kStore, T, U>(acc, it.grad, g_seg, it.grad_elems, c.chunk, g, !whole);
   }
 }
 
@@ -1104,7 +1109,8 @@ typedef void (*publish_fn)(const PublishLaunch);
 
 accum_fn pick_accum(int g, int a, bool store) {  // (gradient dtype, accumulation dtype)
 #define X(E1, T1, E2, T2) \
-  if (g == E1 && a == E2) return store ? accum_kernel<T1, T2, true> : accum_kernel<T1, T2, false>;
+  if (g == E1 && a == E2)                                                            \
+    return store ? accum_kernel<T1, T2, true, kStoreThreads, kStoreUnroll> : accum_kernel<T1, T2, false, kThreads, kUnroll>;
   ODC_FOR_EACH_DTYPE_PAIR(X)
 #undef X
   return nullptr;
@@ -1325,7 +1331,9 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
       blocks_per_cu = L.tt.n_tiles < (uint64_t)opt.accum_persistent_below_tiles * segments ? 1 : 0;
     const uint32_t grid = grid_for(a, blocks_per_cu, L.tt.n_tiles, ragged);
     const int64_t cap = store ? opt.store_resident_cap : opt.accum_resident_cap;
-    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, cap, grid, L.tt.n_tiles), stream, L)) return rc;
+    if (int rc = launch_tiles(a, kernel, grid, lds_claim_for(a, cap, grid, L.tt.n_tiles), stream, L,
+                              store ? kStoreThreads : kThreads))
+      return rc;
   }
   return ODC_OK;
 }
