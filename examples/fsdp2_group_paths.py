@@ -38,6 +38,9 @@ def main():
     ap.add_argument("--publish-groups", type=int, default=0, metavar="K",
                     help="also time the publish of K layer-sized accumulations in ONE launch "
                          "(what pre_optimizer_step does for a model's parameter groups)")
+    ap.add_argument("--compute-dtype-shards", action="store_true",
+                    help="also time the unshard from a bf16 copy of the shards (converted once per "
+                         "minibatch) and that conversion")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="a launch knob of the library, e.g. cast_resident_cap=4")
     args = ap.parse_args()
@@ -55,7 +58,7 @@ def main():
     torch.cuda.set_device(0)
     shapes = [s for _, s in llama3_8b_layer_shapes()]
     N = sum(numel(s) for s in shapes)
-    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * (16 + 4 * args.publish_groups) + (64 << 20))
+    group = odc.init_nvshmem(world_size=W, symmetric_size=(N // W) * (16 + 4 * args.publish_groups + 8 * args.compute_dtype_shards) + (64 << 20))
     fsdp2.patch_fsdp2()  # creates the two services the group uses (nothing of torch is touched here)
     layer = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16,
                              reduce_dtype=torch.float32, name="layer")
@@ -130,6 +133,21 @@ def main():
         ms = timed(lambda: scatter.publish(keys, out_dtype=torch.bfloat16, divisor=float(W)))
         moved = 10 * (N // W) * len(keys)
         print(f"publish of {len(keys)} such groups in one launch: {ms * 1e3:.1f} us, {moved / ms / 1e6:.0f} GB/s")
+    if args.compute_dtype_shards:
+        kept = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16,
+                                name="layer, bf16 copy of the shards", compute_dtype_shards=True)
+        kept.load_full_params([torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes])
+
+        def unshard_kept():
+            kept.unshard()
+            kept.reshard()
+
+        unshard_kept()  # makes the copy
+        gather_ms = timed(unshard_kept)
+        convert_ms = timed(lambda: fsdp2.get_gather_service().convert_symm_buffer(kept.key + "_as_bfloat16", kept.key))
+        print(f"unshard from a bf16 copy of the shards: {gather_ms * 1e3:.1f} us ({4 * N / gather_ms / 1e6:.0f} GB/s); "
+              f"making the copy, once per minibatch, all {W} ranks' shards: {convert_ms * 1e3:.1f} us "
+              f"({6 * N / convert_ms / 1e6:.0f} GB/s)")
     torch.cuda.synchronize()
     fsdp2.stop()
     odc.finalize_distributed()

@@ -56,6 +56,8 @@ def main():
     ap.add_argument("--microbatches", type=int, default=4)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--check", action="store_true")
+    ap.add_argument("--compute-dtype-shards", action="store_true",
+                    help="gather from a bf16 copy of the fp32 shards, converted once per minibatch")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="libodc_hip launch knob, e.g. cast_resident_cap=2")
     args = ap.parse_args()
@@ -85,9 +87,10 @@ def main():
     with torch.device("cuda"):
         model = LlamaForCausalLM(cfg)
     n_params = sum(p.numel() for p in model.parameters())
-    # 4 B shard + 4 B accumulation per parameter and rank, plus room for alignment
-    odc.init_nvshmem(world_size=W, symmetric_size=(n_params // W) * 8 + (64 << 20))
-    fsdp2.patch_fsdp2()
+    # 4 B shard + 4 B accumulation (+ 2 B copy of the shard) per parameter and rank, plus room for alignment
+    per_param = 10 if args.compute_dtype_shards else 8
+    odc.init_nvshmem(world_size=W, symmetric_size=(n_params // W) * per_param + (64 << 20))
+    fsdp2.patch_fsdp2(compute_dtype_shards=args.compute_dtype_shards)
     twin = copy.deepcopy(model).bfloat16()
     for ours, theirs in zip(twin.buffers(), model.buffers()):  # FSDP leaves buffers (rotary) in fp32
         ours.data = theirs.data.clone()
@@ -154,6 +157,9 @@ def main():
     # lm_head) stays unsharded after its forward gather, so it is gathered once
     root_params = n_params - args.layers * layer_params
     path_bytes = args.layers * layer_params * (2 * 6 + 10) + root_params * (6 + 10)
+    if args.compute_dtype_shards:  # gathers move 4 B per element; the copy (6 B) is made once per minibatch
+        path_bytes = (args.layers * layer_params * (2 * 4 + 10) + root_params * (4 + 10)
+                      + 6 * n_params // args.microbatches)
     print(f"Llama {args.layers} x ({args.hidden}, {args.intermediate}) + vocab {args.vocab}: {n_params / 1e6:.0f} M parameters, "
           f"W={W}, {tokens} tokens per microbatch")
     print(f"sharded through ODC : {t_sharded * 1e3:8.2f} ms per microbatch  ({tokens / t_sharded:,.0f} tokens/s)")

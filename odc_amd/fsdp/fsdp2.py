@@ -54,6 +54,8 @@ logger = logging.getLogger(__name__)
 reduction_service = None
 gather_service = None
 _enable_hpz = None
+_compute_dtype_shards = False  # patch_fsdp2(compute_dtype_shards=...)
+_shard_epoch = 0  # bumped by the minibatch hooks: the sharded parameters may have changed since
 
 
 def get_reduction_service():
@@ -133,12 +135,48 @@ def tile_aligned_offsets(numels: Sequence[int], align: int = ACCUMULATION_SLICE_
     return offsets, end
 
 
+def compute_dtype_shards_of(owner, src_key: str, numel: int, dtype: torch.dtype) -> torch.Tensor:
+    """The symmetric buffer ``src_key`` (a group's sharded parameters, ``numel`` elements per
+    rank) converted to ``dtype``, as a second symmetric buffer that is brought up to date before
+    it is returned: the calling rank's view of it, to gather from instead of converting on the way.
+
+    The reference gathers the fp32 shards and casts afterwards (fsdp2.py:341-343); the fused
+    gather here converts on the way (4 + 2 bytes per element and gather). With this copy a gather
+    moves 2 + 2 bytes per element, and the conversion (4 + 2 bytes per element of the shards) is
+    paid once per change of the shards instead of twice per microbatch. It costs the copy's memory:
+    ``numel`` elements of ``dtype`` per rank.
+
+    The copy counts as out of date when a minibatch hook ran since it was made
+    (``pre_minibatch_start``, ``pre_optimizer_step``: the optimizer step lies between them), or
+    when torch has written to any rank's source buffer since (its tensors' version counters; that
+    covers ``load_state_dict``, ``fill_peer_shards`` and in-place optimizers). Code that writes
+    the shards behind torch's back, through raw pointers, must call one of the hooks afterwards.
+    ``owner`` is the object the bookkeeping is kept on."""
+    registry = SymmBufferRegistry.get_instance()
+    key = f"{src_key}_as_{str(dtype).rsplit('.', 1)[-1]}"
+    if not registry.has_key(key):
+        registry.allocate_symm_buffer(key, (numel,), dtype)
+    try:
+        versions = tuple(t._version for t in registry.peer_tensors[src_key])
+    except RuntimeError:  # inference tensors carry no version counter: convert every time
+        versions = None
+    made = owner.__dict__.setdefault("_odc_compute_dtype_shards", {})
+    stamp = (versions, _shard_epoch)
+    if versions is None or made.get(key) != stamp:
+        get_gather_service().convert_symm_buffer(key, src_key)
+        made[key] = stamp
+    return registry.get_symm_buffer(key)
+
+
 class ParamGroup:
     """One FSDP2 parameter group in the symmetric arena, as seen by the calling rank."""
 
     def __init__(self, shapes, dtype: torch.dtype, pg, param_dtype: Optional[torch.dtype] = None,
-                 reduce_dtype: Optional[torch.dtype] = None, reduce_op: str = "avg", name: str = ""):
+                 reduce_dtype: Optional[torch.dtype] = None, reduce_op: str = "avg", name: str = "",
+                 compute_dtype_shards: bool = False):
         self.shapes = [tuple(s) for s in shapes]
+        # keep a copy of the shards in param_dtype and gather from it (compute_dtype_shards_of)
+        self.compute_dtype_shards = compute_dtype_shards
         self.dtype = dtype              # dtype of the sharded parameters (orig dtype)
         self.param_dtype = param_dtype  # dtype the unsharded parameters are used in (None = dtype)
         self.reduce_dtype = reduce_dtype
@@ -201,7 +239,10 @@ class ParamGroup:
         if fused:
             # straight into per-parameter buffers, converted to the compute dtype on the way
             padded = [torch.empty(W * n, dtype=out_dtype, device=device) for n in self.shard_numels]
-            gather.gather_slices(padded, self.symm_buffer, self.offsets, self.shard_numels, self.pg)
+            source = self.symm_buffer
+            if self.compute_dtype_shards and out_dtype != self.dtype:
+                source = compute_dtype_shards_of(self, self.key, self.total_shard_numel, out_dtype)
+            gather.gather_slices(padded, source, self.offsets, self.shard_numels, self.pg)
         else:
             padded = [torch.empty(W * n, dtype=self.dtype, device=device) for n in self.shard_numels]
             ag = torch.empty(W * self.total_shard_numel, dtype=self.dtype, device=device)
@@ -427,7 +468,10 @@ def foreach_all_gather(fsdp_params, group, async_op, all_gather_copy_in_stream, 
             numels.append(n)
             dtypes_meta.append([out_dtype])
             numels_meta.append([n])
-        get_gather_service().gather_slices(outs, fsdp_group._odc_symm_buffer, offsets, numels, group)
+        source = fsdp_group._odc_symm_buffer
+        if _compute_dtype_shards and out_dtype != layout.dtype:
+            source = compute_dtype_shards_of(fsdp_group, layout.key, layout.total, out_dtype)
+        get_gather_service().gather_slices(outs, source, offsets, numels, group)
         all_gather_event = all_gather_stream.record_event()
     placeholder = torch.empty(0, dtype=out_dtype, device=device)
     return AllGatherResult(placeholder, all_gather_event, None, dtypes_meta, numels_meta, numels)
@@ -614,6 +658,8 @@ def _param_groups(fsdp_module) -> List[ParamGroup]:
 
 def pre_minibatch_start(fsdp_module):
     """fsdp2.py:427-433 (without the HPZ reshard)."""
+    global _shard_epoch
+    _shard_epoch += 1  # copies of the shards in the compute dtype are made anew
     get_reduction_service().clear_accumulations()
     if torch.distributed.is_available() and torch.distributed.is_initialized():
         torch.distributed.barrier()
@@ -621,6 +667,8 @@ def pre_minibatch_start(fsdp_module):
 
 def pre_optimizer_step(fsdp_module):
     """fsdp2.py:1023-1046: sync once, then publish every group's gradients."""
+    global _shard_epoch
+    _shard_epoch += 1  # the optimizer is about to change the shards
     scatter = get_reduction_service()
     if _is_torch_fsdp_module(fsdp_module):
         groups = _torch_param_groups(fsdp_module)
@@ -655,13 +703,20 @@ def _comm_context_lazy_init(self, device):
         self.reduce_scatter_stream = self.device_handle.Stream()
 
 
-def patch_fsdp2(enable_hpz: bool = False) -> None:
+def patch_fsdp2(enable_hpz: bool = False, compute_dtype_shards: Optional[bool] = None) -> None:
     """Create the two services and route torch's fully_shard collectives through them
-    (fsdp2.py:1105-1138). Modules sharded afterwards need ``patch_lazy_init(module)`` each."""
-    global _enable_hpz, reduction_service, gather_service
+    (fsdp2.py:1105-1138). Modules sharded afterwards need ``patch_lazy_init(module)`` each.
+
+    ``compute_dtype_shards`` (default: ``$ODC_FSDP2_COMPUTE_DTYPE_SHARDS == "1"``, off): under a
+    mixed-precision policy, keep every group's shards a second time in ``param_dtype`` and gather
+    from that copy (``compute_dtype_shards_of``)."""
+    global _enable_hpz, reduction_service, gather_service, _compute_dtype_shards
     if enable_hpz:
         raise NotImplementedError("HPZ needs more than one node; not part of this build")
     _enable_hpz = False
+    if compute_dtype_shards is None:
+        compute_dtype_shards = os.environ.get("ODC_FSDP2_COMPUTE_DTYPE_SHARDS", "0") == "1"
+    _compute_dtype_shards = bool(compute_dtype_shards)
     from torch.distributed.fsdp._fully_shard import _fsdp_collectives, _fsdp_param_group
 
     comm_context = _fsdp_param_group.FSDPCommContext

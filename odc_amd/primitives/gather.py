@@ -174,3 +174,39 @@ class GatherService:
                 numels.append(n)
         if outs:
             self._gather(outs, offsets, numels, input_tensor.dtype, pg)
+
+    def convert_symm_buffer(self, dst_key, src_key, ranks: Sequence[int] = None) -> None:
+        """Rank r's symmetric buffer ``dst_key`` = rank r's ``src_key`` converted to the
+        destination's dtype (round to nearest even), for every rank whose memory this process
+        holds (``ranks`` narrows it; with one process per GPU a rank converts its own shard).
+        One launch per rank, on the launch stream of the other primitives.
+
+        It is what keeps a copy of the sharded parameters in the compute dtype: converted once
+        after the optimizer step (4 + 2 bytes per element of ONE shard), so that every gather of
+        the minibatch moves 2 + 2 bytes per element instead of converting on the way (4 + 2),
+        the FSDP2 counterpart of the copy-once-until-flush of ``odc/primitives/utils.py:103-116``
+        that ``odc/fsdp/fsdp1.py:239-247`` uses for the low-precision shard."""
+        registry = SymmBufferRegistry.get_instance()
+        world = get_world()
+        src_offset, src_shape, src_dtype = registry.offsets[src_key]
+        _dst_offset, dst_shape, dst_dtype = registry.offsets[dst_key]
+        assert tuple(src_shape) == tuple(dst_shape), f"{src_key}: {src_shape} != {dst_key}: {dst_shape}"
+        numel = 1
+        for d in src_shape:
+            numel *= d
+        if not numel:
+            return
+        item = (_native.PublishItem * 1)()
+        item[0].acc_offset = src_offset
+        item[0].elems = numel
+        lib = _native.load()
+        peers = registry.peer_tensors[dst_key]
+        with comm_stream_section("odc.convert") as comm:
+            stream = ctypes.c_void_p(comm.cuda_stream)
+            for r in range(world.world_size) if ranks is None else ranks:
+                item[0].out = peers[r].data_ptr()
+                _native.check(
+                    lib.odc_publish(
+                        world.arena.handle, r, item, 1, native_dtype(src_dtype), native_dtype(dst_dtype), 1.0, stream
+                    )
+                )

@@ -136,6 +136,65 @@ def test_fsdp2_group_layout(make_world, W, fused, dtype):
     assert not utils.is_initialized()
 
 
+def test_fsdp2_group_gathers_from_shards_kept_in_the_compute_dtype(make_world):
+    """fp32 shards, bf16 compute, ``compute_dtype_shards=True``: the group keeps a bf16 copy of
+    every rank's shards, converts it once per change of the shards and gathers from it. The
+    unsharded parameters are bit-equal to converting on the way; an in-place update through torch
+    is seen without any hook; one that bypasses torch's version counters is seen after the hook."""
+    from odc_amd import SymmBufferRegistry
+    from odc_amd.fsdp import fsdp2
+
+    W = 4
+    group = make_world(W, 32 << 20)
+    fsdp2.patch_fsdp2()
+    shapes = [(37, 24), (5,), (1024, 96), (W + 1, 33)]
+    g = torch.Generator().manual_seed(5)
+    params = [torch.randn(*s, generator=g) * 0.02 for s in shapes]
+    kept = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16, compute_dtype_shards=True)
+    plain = fsdp2.ParamGroup(shapes, torch.float32, group, param_dtype=torch.bfloat16)
+    for pgp in (kept, plain):
+        pgp.load_full_params([p.cuda() for p in params])
+    service = fsdp2.get_gather_service()
+    conversions = []
+    convert = service.convert_symm_buffer
+    service.convert_symm_buffer = lambda *a, **k: (conversions.append(a), convert(*a, **k))[1]
+
+    def check(what, n_conversions):
+        for _ in range(3):  # three unshards, one conversion
+            got = kept.unshard()
+        want = plain.unshard()
+        for p, (a, b) in enumerate(zip(got, want)):
+            assert a.dtype == torch.bfloat16
+            assert_bit_equal(a, b, f"{what}: unsharded param {p}")
+        assert len(conversions) == n_conversions, what
+        return got
+
+    got = check("fresh", 1)
+    for p, full in enumerate(params):
+        assert_bit_equal(got[p], full.to(torch.bfloat16), f"unsharded param {p} vs original")
+    registry = SymmBufferRegistry.get_instance()
+    copy_key = kept.key + "_as_bfloat16"
+    assert registry.has_key(copy_key) and registry.offsets[copy_key][2] == torch.bfloat16
+    assert not registry.has_key(plain.key + "_as_bfloat16")
+
+    # an optimizer step through torch (in place, on every rank's shards): seen by the version counters
+    for pgp in (kept, plain):
+        for r in range(W):
+            for shard in pgp.sharded_params(r):
+                shard.mul_(1.5).add_(0.001)
+    check("after an in-place update", 2)
+    check("unchanged shards", 2)
+
+    # a write that torch's version counters do not see: the minibatch hook makes the copy anew
+    for pgp in (kept, plain):
+        for buf in registry.peer_tensors[pgp.key]:
+            buf.data.mul_(-0.5)
+    fsdp2.pre_minibatch_start(types.SimpleNamespace(_odc_param_groups=[kept, plain]))
+    check("after the hook", 3)
+    del got
+    fsdp2.stop()
+
+
 def test_group_paths_example_runs():
     """examples/fsdp2_group_paths.py (reference data flow against the fused one, timed) runs to
     the end; equality of the two flows is what test_fsdp2_group_layout checks."""

@@ -66,10 +66,13 @@ def fake_process_group():
 
 @pytest.mark.parametrize("dims", [(96, 50), (192, 1100)], ids=["small", "wide"])
 @pytest.mark.parametrize("W", [4, 8])
-@pytest.mark.parametrize("mixed", [True, False])
+@pytest.mark.parametrize("mixed", [True, False, "compute-dtype shards"])
 def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_group, W, mixed, dims):
     """`wide`: the weight shards exceed one tile (4096 elements), so the groups' accumulations
-    have their slices on tile boundaries, with gaps after the small ones (norms, biases)."""
+    have their slices on tile boundaries, with gaps after the small ones (norms, biases).
+    `compute-dtype shards`: mixed precision with the gathers reading a bf16 copy of the shards
+    that is converted once per minibatch; the forward after the optimizer step must see the
+    updated shards."""
     from torch.distributed.device_mesh import init_device_mesh
     from torch.distributed.fsdp import MixedPrecisionPolicy, fully_shard
 
@@ -78,7 +81,7 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
     fake_process_group(W)
     mesh = init_device_mesh("cuda", (W,))
     make_world(W, 64 << 20)
-    fsdp2.patch_fsdp2()
+    fsdp2.patch_fsdp2(compute_dtype_shards=mixed == "compute-dtype shards")
 
     torch.manual_seed(0)
     model = Toy(dim=dims[0], hidden=dims[1]).cuda()
@@ -101,6 +104,9 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
         fsdp2.fill_peer_shards(module, full_params)
     breakdown = fsdp2.get_symm_buffer_memory_breakdown()
     assert set(breakdown) >= {"fsdp_params", "accumulation"}
+    conversions = []
+    convert = fsdp2.get_gather_service().convert_symm_buffer
+    fsdp2.get_gather_service().convert_symm_buffer = lambda *a, **k: (conversions.append(a), convert(*a, **k))[1]
     # rank 0's shard of every parameter is chunk 0 of the full parameter, living in the arena
     for name, p in model.named_parameters():
         local = p._local_tensor
@@ -153,6 +159,9 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
             p[:rows] = updated[name]
     want_out = copy.deepcopy(reference).to(compute_dtype)(batches[0].to(compute_dtype))
     assert_bit_equal(out, want_out, "forward after the optimizer step")
+    # one conversion per group and minibatch, however many gathers (forward and backward, M microbatches)
+    n_groups = len(model.layers) + 1
+    assert len(conversions) == (2 * n_groups if mixed == "compute-dtype shards" else 0)
 
 
 @pytest.mark.parametrize("extra", [
