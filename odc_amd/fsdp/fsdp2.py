@@ -135,7 +135,8 @@ def tile_aligned_offsets(numels: Sequence[int], align: int = ACCUMULATION_SLICE_
     return offsets, end
 
 
-def compute_dtype_shards_of(owner, src_key: str, numel: int, dtype: torch.dtype) -> torch.Tensor:
+def compute_dtype_shards_of(owner, src_key: str, numel: int, dtype: torch.dtype,
+                            watch: Sequence[torch.Tensor] = ()) -> torch.Tensor:
     """The symmetric buffer ``src_key`` (a group's sharded parameters, ``numel`` elements per
     rank) converted to ``dtype``, as a second symmetric buffer that is brought up to date before
     it is returned: the calling rank's view of it, to gather from instead of converting on the way.
@@ -148,16 +149,18 @@ def compute_dtype_shards_of(owner, src_key: str, numel: int, dtype: torch.dtype)
 
     The copy counts as out of date when a minibatch hook ran since it was made
     (``pre_minibatch_start``, ``pre_optimizer_step``: the optimizer step lies between them), or
-    when torch has written to any rank's source buffer since (its tensors' version counters; that
-    covers ``load_state_dict``, ``fill_peer_shards`` and in-place optimizers). Code that writes
-    the shards behind torch's back, through raw pointers, must call one of the hooks afterwards.
-    ``owner`` is the object the bookkeeping is kept on."""
+    when torch has written to the shards since: the version counters of every rank's source
+    buffer (writes through views of it: ``fill_peer_shards``, ``load_full_params``) and of the
+    tensors in ``watch`` — the sharded parameters themselves, whose in-place updates as DTensors
+    (optimizers, ``load_state_dict``) bump the DTensor's counter, not its local tensor's. Code that
+    writes the shards behind torch's back, through raw pointers, must call one of the hooks
+    afterwards. ``owner`` is the object the bookkeeping is kept on."""
     registry = SymmBufferRegistry.get_instance()
     key = f"{src_key}_as_{str(dtype).rsplit('.', 1)[-1]}"
     if not registry.has_key(key):
         registry.allocate_symm_buffer(key, (numel,), dtype)
     try:
-        versions = tuple(t._version for t in registry.peer_tensors[src_key])
+        versions = tuple(t._version for t in (*registry.peer_tensors[src_key], *watch))
     except RuntimeError:  # inference tensors carry no version counter: convert every time
         versions = None
     made = owner.__dict__.setdefault("_odc_compute_dtype_shards", {})
@@ -470,7 +473,8 @@ def foreach_all_gather(fsdp_params, group, async_op, all_gather_copy_in_stream, 
             numels_meta.append([n])
         source = fsdp_group._odc_symm_buffer
         if _compute_dtype_shards and out_dtype != layout.dtype:
-            source = compute_dtype_shards_of(fsdp_group, layout.key, layout.total, out_dtype)
+            source = compute_dtype_shards_of(fsdp_group, layout.key, layout.total, out_dtype,
+                                             watch=[fp.sharded_param for fp in fsdp_group.fsdp_params])
         get_gather_service().gather_slices(outs, source, offsets, numels, group)
         all_gather_event = all_gather_stream.record_event()
     placeholder = torch.empty(0, dtype=out_dtype, device=device)

@@ -162,6 +162,19 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
     # one conversion per group and minibatch, however many gathers (forward and backward, M microbatches)
     n_groups = len(model.layers) + 1
     assert len(conversions) == (2 * n_groups if mixed == "compute-dtype shards" else 0)
+    if mixed == "compute-dtype shards":
+        # an in-place update of the sharded parameters with no hook in between (a checkpoint
+        # load, say): torch's version counters tell the copies that they are out of date
+        model.reshard()
+        with torch.no_grad():
+            for p in model.parameters():
+                p.mul_(0.5)
+            for p in reference.parameters():
+                p[: math.ceil(p.shape[0] / W)].mul_(0.5)
+        out = model(batches[1])
+        want_out = copy.deepcopy(reference).to(compute_dtype)(batches[1].to(compute_dtype))
+        assert_bit_equal(out, want_out, "forward after an in-place update without a hook")
+        assert len(conversions) == 3 * n_groups
 
 
 @pytest.mark.parametrize("extra", [
