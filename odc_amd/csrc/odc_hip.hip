@@ -77,9 +77,10 @@ int fail(int code, const char* fmt, ...) {
 // 20 %). The read-modify-write keeps 256 x 4 (512 x 2: equal on long segments, -3 % in the
 // persistent shape at W=64), and so does the clear (512 x 2: -25 % on per-parameter spans).
 constexpr int kCopyThreads = 512;
-constexpr int kCopyUnroll = 2;
+constexpr int kCopyUnroll = (int)odc_tiles::kTileVecs / kCopyThreads;  // 2 for the 16 KiB tile
 constexpr int kStoreThreads = 512;
-constexpr int kStoreUnroll = 2;
+constexpr int kStoreUnroll = (int)odc_tiles::kTileVecs / kStoreThreads;
+static_assert(kCopyUnroll >= 1 && kStoreUnroll >= 1, "a tile holds at least one vector per thread");
 
 struct Options {
   // measured on MI355X over a Llama-3-8B layer: every kernel peaks with one workgroup per tile
