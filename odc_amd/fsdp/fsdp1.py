@@ -19,17 +19,20 @@ process group (for instance torch's "fake" backend).
 from __future__ import annotations
 
 import logging
+import os
 
 import torch
 import torch.nn.functional as F
 
 import odc_amd
+from odc_amd.fsdp.shard_copies import compute_dtype_shards_of, shards_may_have_changed
 from odc_amd.primitives.utils import group_size
 
 logger = logging.getLogger(__name__)
 
 reduction_service = None
 gather_service = None
+_compute_dtype_shards = False  # patch_fsdp1(compute_dtype_shards=...)
 
 
 def get_reduction_service():
@@ -64,17 +67,26 @@ def get_shard(tensor: torch.Tensor, rank: int, world_size: int):
 custom_get_shard = get_shard  # the reference's name for it (fsdp1.py:239)
 
 
-def all_gather_flat_param(padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=None):
+def all_gather_flat_param(padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=None, watch=()):
     """Gather the padded flat parameter. The shards stay in their own dtype (a peer may not have
     produced a low-precision copy yet: that is why the reference gathers in the shard dtype into
     a temporary and casts afterwards, fsdp1.py:199-223); when the output dtype differs, the
-    conversion happens inside the gather kernel."""
+    conversion happens inside the gather kernel, or, with ``patch_fsdp1(compute_dtype_shards=True)``,
+    once per change of the shards into a copy that the gathers then read
+    (``shard_copies.compute_dtype_shards_of``; ``watch``: the flat parameter, whose version
+    counter the optimizer bumps)."""
     expected = sharded_flat_param.numel() * group_size(pg)
     assert (
         padded_unsharded_flat_param.numel() == expected
     ), f"Expects {expected} numel but got {padded_unsharded_flat_param.numel()}"
     if padded_unsharded_flat_param.dtype != sharded_flat_param.dtype:
         assert param_dtype in (None, padded_unsharded_flat_param.dtype)
+        if _compute_dtype_shards and sharded_flat_param.numel():
+            registry = odc_amd.SymmBufferRegistry.get_instance()
+            key = registry.local_tensor_to_keys[sharded_flat_param.data_ptr()]
+            sharded_flat_param = compute_dtype_shards_of(
+                gather_service, key, sharded_flat_param.numel(), padded_unsharded_flat_param.dtype, watch=watch
+            )
     gather_service.gather_into_tensor(padded_unsharded_flat_param, sharded_flat_param, pg)
     return padded_unsharded_flat_param
 
@@ -137,7 +149,8 @@ def _patched_all_gather_flat_param(self, padded_unsharded_flat_param):
     pg = self._fake_process_group if self._use_fake_all_gather else self.process_group
     assert not sharded_flat_param.is_cpu and not self._offload_params, "ODC does not support offloading"
     return all_gather_flat_param(
-        padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=self._fwd_bwd_param_dtype
+        padded_unsharded_flat_param, sharded_flat_param, pg, param_dtype=self._fwd_bwd_param_dtype,
+        watch=(self.flat_param,),
     )
 
 
@@ -183,11 +196,18 @@ def _patched_prepare_gradient_for_optim(self):
         delattr(flat_param, "_saved_grad_shard")
 
 
-def patch_fsdp1(reduce_dtype=None):
+def patch_fsdp1(reduce_dtype=None, compute_dtype_shards=None):
     """Create the two services and route torch FSDP1's all-gather and reduce-scatter through
     them (fsdp1.py:302-314). Call before wrapping modules: shards move into the symmetric arena
-    when ``FullyShardedDataParallel`` shards its flat parameters."""
-    global reduction_service, gather_service
+    when ``FullyShardedDataParallel`` shards its flat parameters.
+
+    ``compute_dtype_shards`` (default: ``$ODC_FSDP1_COMPUTE_DTYPE_SHARDS == "1"``, off): under
+    mixed precision, keep every flat parameter's shards a second time in the compute dtype and
+    gather from that copy."""
+    global reduction_service, gather_service, _compute_dtype_shards
+    if compute_dtype_shards is None:
+        compute_dtype_shards = os.environ.get("ODC_FSDP1_COMPUTE_DTYPE_SHARDS", "0") == "1"
+    _compute_dtype_shards = bool(compute_dtype_shards)
     reduction_service = odc_amd.ReductionService(accumulation_dtype=reduce_dtype)
     gather_service = odc_amd.GatherService()
     from torch.distributed.fsdp import _runtime_utils
@@ -227,6 +247,7 @@ def unpatch_fsdp1():
 def pre_optimizer_step(fsdp_module):
     """fsdp1.py:317-335: wait for every add, post-divide, publish the accumulations as
     ``flat_param.grad`` in the parameter dtype."""
+    shards_may_have_changed()  # the optimizer is about to change them
     with torch.cuda.nvtx.range("scatter_accumulate_sync"):
         get_reduction_service().sync(getattr(fsdp_module, "process_group", None))
     if hasattr(fsdp_module, "_inter_node_pg"):
@@ -258,6 +279,7 @@ def pre_optimizer_step(fsdp_module):
 def pre_minibatch_start(_fsdp_module):
     """fsdp1.py:338-342: zero the accumulations; the reference then barriers so that optimizer
     updates are visible to all ranks, which for ranks sharing one device is stream order."""
+    shards_may_have_changed()
     get_reduction_service().clear_accumulations()
     if torch.distributed.is_available() and torch.distributed.is_initialized():
         torch.distributed.barrier()

@@ -40,6 +40,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
+from odc_amd.fsdp.shard_copies import compute_dtype_shards_of, shards_may_have_changed
 from odc_amd.primitives.gather import GatherService
 from odc_amd.primitives.scatter_accumulate import ReductionService
 from odc_amd.primitives.utils import (
@@ -55,7 +56,6 @@ reduction_service = None
 gather_service = None
 _enable_hpz = None
 _compute_dtype_shards = False  # patch_fsdp2(compute_dtype_shards=...)
-_shard_epoch = 0  # bumped by the minibatch hooks: the sharded parameters may have changed since
 
 
 def get_reduction_service():
@@ -135,42 +135,6 @@ def tile_aligned_offsets(numels: Sequence[int], align: int = ACCUMULATION_SLICE_
     return offsets, end
 
 
-def compute_dtype_shards_of(owner, src_key: str, numel: int, dtype: torch.dtype,
-                            watch: Sequence[torch.Tensor] = ()) -> torch.Tensor:
-    """The symmetric buffer ``src_key`` (a group's sharded parameters, ``numel`` elements per
-    rank) converted to ``dtype``, as a second symmetric buffer that is brought up to date before
-    it is returned: the calling rank's view of it, to gather from instead of converting on the way.
-
-    The reference gathers the fp32 shards and casts afterwards (fsdp2.py:341-343); the fused
-    gather here converts on the way (4 + 2 bytes per element and gather). With this copy a gather
-    moves 2 + 2 bytes per element, and the conversion (4 + 2 bytes per element of the shards) is
-    paid once per change of the shards instead of twice per microbatch. It costs the copy's memory:
-    ``numel`` elements of ``dtype`` per rank.
-
-    The copy counts as out of date when a minibatch hook ran since it was made
-    (``pre_minibatch_start``, ``pre_optimizer_step``: the optimizer step lies between them), or
-    when torch has written to the shards since: the version counters of every rank's source
-    buffer (writes through views of it: ``fill_peer_shards``, ``load_full_params``) and of the
-    tensors in ``watch`` — the sharded parameters themselves, whose in-place updates as DTensors
-    (optimizers, ``load_state_dict``) bump the DTensor's counter, not its local tensor's. Code that
-    writes the shards behind torch's back, through raw pointers, must call one of the hooks
-    afterwards. ``owner`` is the object the bookkeeping is kept on."""
-    registry = SymmBufferRegistry.get_instance()
-    key = f"{src_key}_as_{str(dtype).rsplit('.', 1)[-1]}"
-    if not registry.has_key(key):
-        registry.allocate_symm_buffer(key, (numel,), dtype)
-    try:
-        versions = tuple(t._version for t in (*registry.peer_tensors[src_key], *watch))
-    except RuntimeError:  # inference tensors carry no version counter: convert every time
-        versions = None
-    made = owner.__dict__.setdefault("_odc_compute_dtype_shards", {})
-    stamp = (versions, _shard_epoch)
-    if versions is None or made.get(key) != stamp:
-        get_gather_service().convert_symm_buffer(key, src_key)
-        made[key] = stamp
-    return registry.get_symm_buffer(key)
-
-
 class ParamGroup:
     """One FSDP2 parameter group in the symmetric arena, as seen by the calling rank."""
 
@@ -244,7 +208,7 @@ class ParamGroup:
             padded = [torch.empty(W * n, dtype=out_dtype, device=device) for n in self.shard_numels]
             source = self.symm_buffer
             if self.compute_dtype_shards and out_dtype != self.dtype:
-                source = compute_dtype_shards_of(self, self.key, self.total_shard_numel, out_dtype)
+                source = compute_dtype_shards_of(gather, self.key, self.total_shard_numel, out_dtype)
             gather.gather_slices(padded, source, self.offsets, self.shard_numels, self.pg)
         else:
             padded = [torch.empty(W * n, dtype=self.dtype, device=device) for n in self.shard_numels]
@@ -473,7 +437,7 @@ def foreach_all_gather(fsdp_params, group, async_op, all_gather_copy_in_stream, 
             numels_meta.append([n])
         source = fsdp_group._odc_symm_buffer
         if _compute_dtype_shards and out_dtype != layout.dtype:
-            source = compute_dtype_shards_of(fsdp_group, layout.key, layout.total, out_dtype,
+            source = compute_dtype_shards_of(get_gather_service(), layout.key, layout.total, out_dtype,
                                              watch=[fp.sharded_param for fp in fsdp_group.fsdp_params])
         get_gather_service().gather_slices(outs, source, offsets, numels, group)
         all_gather_event = all_gather_stream.record_event()
@@ -662,8 +626,7 @@ def _param_groups(fsdp_module) -> List[ParamGroup]:
 
 def pre_minibatch_start(fsdp_module):
     """fsdp2.py:427-433 (without the HPZ reshard)."""
-    global _shard_epoch
-    _shard_epoch += 1  # copies of the shards in the compute dtype are made anew
+    shards_may_have_changed()  # copies of the shards in the compute dtype are made anew
     get_reduction_service().clear_accumulations()
     if torch.distributed.is_available() and torch.distributed.is_initialized():
         torch.distributed.barrier()
@@ -671,8 +634,7 @@ def pre_minibatch_start(fsdp_module):
 
 def pre_optimizer_step(fsdp_module):
     """fsdp2.py:1023-1046: sync once, then publish every group's gradients."""
-    global _shard_epoch
-    _shard_epoch += 1  # the optimizer is about to change the shards
+    shards_may_have_changed()  # the optimizer is about to change the shards
     scatter = get_reduction_service()
     if _is_torch_fsdp_module(fsdp_module):
         groups = _torch_param_groups(fsdp_module)

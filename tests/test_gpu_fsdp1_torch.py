@@ -40,8 +40,12 @@ def fake_process_group():
         dist.destroy_process_group()
 
 
+@pytest.mark.parametrize("shard_copies", [False, True], ids=["converting gather", "compute-dtype shards"])
 @pytest.mark.parametrize("W", [4, 8])
-def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, W):
+def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, W, shard_copies):
+    """``compute-dtype shards``: the gathers read a bf16 copy of the fp32 shards that is converted
+    once per minibatch; the forward after the optimizer step must see the updated shards, with
+    and without a hook in between."""
     from torch.distributed.fsdp import FullyShardedDataParallel as FSDP
     from torch.distributed.fsdp import MixedPrecision
     from torch.distributed.fsdp._common_utils import clean_tensor_name
@@ -52,7 +56,11 @@ def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, 
 
     fake_process_group(W)
     group = make_world(W, 64 << 20)
-    fsdp1.patch_fsdp1(reduce_dtype=torch.float32)  # bf16 gradients into fp32 accumulations
+    # bf16 gradients into fp32 accumulations
+    fsdp1.patch_fsdp1(reduce_dtype=torch.float32, compute_dtype_shards=shard_copies)
+    conversions = []
+    convert = fsdp1.get_gather_service().convert_symm_buffer
+    fsdp1.get_gather_service().convert_symm_buffer = lambda *a, **k: (conversions.append(a), convert(*a, **k))[1]
 
     torch.manual_seed(0)
     model = Toy().cuda()
@@ -122,6 +130,25 @@ def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, 
                 off += named[f].numel()
     want_out = copy.deepcopy(reference).bfloat16()(batches[0].bfloat16())
     assert_bit_equal(out, want_out, "forward after the optimizer step")
+    # one conversion per unit and minibatch, however many gathers
+    assert len(conversions) == (2 * len(units) if shard_copies else 0)
+    if shard_copies:
+        # an in-place update with no hook in between: the flat parameters' version counters tell
+        out.float().pow(2).mean().backward()  # leaves every unit resharded, the root's too
+        with torch.no_grad():
+            for handle, fqns in units:
+                handle.flat_param.mul_(0.5)
+                flat = torch.cat([named[f].reshape(-1) for f in fqns])
+                S = math.ceil(flat.numel() / W)
+                flat[:S] = handle.flat_param.data[: min(S, flat.numel())]
+                off = 0
+                for f in fqns:
+                    named[f].copy_(flat[off : off + named[f].numel()].view_as(named[f]))
+                    off += named[f].numel()
+        out = fsdp_model(batches[1])
+        want_out = copy.deepcopy(reference).bfloat16()(batches[1].bfloat16())
+        assert_bit_equal(out, want_out, "forward after an in-place update without a hook")
+        assert len(conversions) == 3 * len(units)
 
 
 @pytest.mark.parametrize("extra", [
