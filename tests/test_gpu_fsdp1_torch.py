@@ -156,6 +156,7 @@ def test_fsdp1_minibatch_through_the_primitives(make_world, fake_process_group, 
     ["--world-size", "5", "--layers", "2", "--no-backward-prefetch", "--microbatches", "3"],
     ["--world-size", "12", "--layers", "3", "--shard-grad-op"],
     ["--world-size", "8", "--layers", "2", "--microbatches", "4", "--sync-every", "2"],
+    ["--world-size", "12", "--layers", "3", "--forward-prefetch", "ENV:ODC_FSDP1_COMPUTE_DTYPE_SHARDS=1"],
 ])
 def test_transformer_example_trains_bit_exactly(extra):
     """examples/fsdp1_toy.py: a small transformer under FSDP1 with forward / backward prefetching
@@ -165,8 +166,13 @@ def test_transformer_example_trains_bit_exactly(extra):
     from pathlib import Path
 
     script = Path(__file__).resolve().parent.parent / "examples" / "fsdp1_toy.py"
-    proc = subprocess.run([sys.executable, str(script), "--steps", "3", *extra],
-                          capture_output=True, text=True, timeout=300)
+    import os
+
+    env = dict(os.environ)
+    env.update(e[4:].split("=", 1) for e in extra if e.startswith("ENV:"))
+    args = [e for e in extra if not e.startswith("ENV:")]
+    proc = subprocess.run([sys.executable, str(script), "--steps", "3", *args],
+                          capture_output=True, text=True, timeout=300, env=env)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert proc.stdout.count("match the unsharded model bit for bit") == 3
 

@@ -186,6 +186,8 @@ def test_fully_shard_minibatch_through_the_primitives(make_world, fake_process_g
     ["--world-size", "12", "--layers", "2", "--mixed-precision", "--reduce-dtype", "fp16", "--microbatches", "4",
      "--sync-every", "2"],  # pre- and post-divide around fp16 accumulations
     ["--world-size", "8", "--layers", "2", "--mixed-precision", "--reduce-dtype", "bf16", "--microbatches", "3"],
+    ["--world-size", "12", "--layers", "3", "--mixed-precision", "--explicit-prefetching",
+     "ENV:ODC_FSDP2_COMPUTE_DTYPE_SHARDS=1"],  # gathers read a bf16 copy of the shards, renewed every step
 ])
 def test_transformer_example_trains_bit_exactly(extra):
     """examples/fsdp2_toy.py (the counterpart of examples/FSDP2/example.py): a small transformer
@@ -197,8 +199,13 @@ def test_transformer_example_trains_bit_exactly(extra):
     from pathlib import Path
 
     script = Path(__file__).resolve().parent.parent / "examples" / "fsdp2_toy.py"
-    proc = subprocess.run([sys.executable, str(script), "--steps", "4", *extra],
-                          capture_output=True, text=True, timeout=300)
+    import os
+
+    env = dict(os.environ)
+    env.update(e[4:].split("=", 1) for e in extra if e.startswith("ENV:"))
+    args = [e for e in extra if not e.startswith("ENV:")]
+    proc = subprocess.run([sys.executable, str(script), "--steps", "4", *args],
+                          capture_output=True, text=True, timeout=300, env=env)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     assert proc.stdout.count("match the unsharded model bit for bit") == 4
 
