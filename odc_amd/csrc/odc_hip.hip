@@ -1079,6 +1079,16 @@ int check_rank_range(const odc_arena* a, const char* what, uint32_t i, uint64_t 
   return ODC_OK;
 }
 
+// The same for `elems` elements of `elem_bytes` each; an element count whose byte size would wrap
+// around is rejected before it is multiplied.
+int check_rank_elems(const odc_arena* a, const char* what, uint32_t i, uint64_t offset, uint64_t elems,
+                     uint64_t elem_bytes) {
+  if (elems > a->bytes_per_rank / elem_bytes)
+    return fail(ODC_ERR_INVALID, "%s %u: %llu elements of %llu bytes exceed the %llu byte rank region", what, i,
+                (unsigned long long)elems, (unsigned long long)elem_bytes, (unsigned long long)a->bytes_per_rank);
+  return check_rank_range(a, what, i, offset, elems * elem_bytes);
+}
+
 // dst [d0, d0 + world*seg_bytes) must not overlap any rank's source range at src_offset.
 int check_no_overlap(const odc_arena* a, uint32_t i, const void* dst, uint64_t dst_seg_bytes,
                      uint64_t src_offset, uint64_t src_seg_bytes) {
@@ -1195,7 +1205,7 @@ int odc_gather_cast(odc_arena* a, const odc_gather_cast_item* items, uint32_t n_
                   (unsigned long long)it.shard_elems);
     if (it.src_offset % sb || (uintptr_t)it.dst % db)
       return fail(ODC_ERR_INVALID, "item %u: src_offset or dst is not aligned to its dtype", i);
-    if (int rc = check_rank_range(a, "item", i, it.src_offset, it.shard_elems * sb)) return rc;
+    if (int rc = check_rank_elems(a, "item", i, it.src_offset, it.shard_elems, sb)) return rc;
     if (int rc = check_no_overlap(a, i, it.dst, it.shard_elems * db, it.src_offset, it.shard_elems * sb)) return rc;
   }
   const Options opt = options_snapshot();
@@ -1276,7 +1286,7 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     if (it.acc_offset % ab)
       return fail(ODC_ERR_INVALID, "item %u: acc_offset %llu is not aligned to the accumulation dtype", i,
                   (unsigned long long)it.acc_offset);
-    if (int rc = check_rank_range(a, "item", i, it.acc_offset, it.shard_elems * ab)) return rc;
+    if (int rc = check_rank_elems(a, "item", i, it.acc_offset, it.shard_elems, ab)) return rc;
     if (it.grad_elems > it.shard_elems * a->world)
       return fail(ODC_ERR_INVALID, "item %u: grad_elems %llu > world_size * shard_elems = %llu", i,
                   (unsigned long long)it.grad_elems, (unsigned long long)(it.shard_elems * a->world));

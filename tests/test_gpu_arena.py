@@ -91,6 +91,22 @@ def test_arena_exhaustion_and_bad_arguments(make_world):
     item[0].shard_bytes = 32
     assert lib.odc_gather(arena.handle, item, 1, 0, None) == _native.ODC_ERR_INVALID
     assert b"overlaps" in lib.odc_last_error()
+    # element counts whose byte size wraps around 2**64 are refused like any other overrun
+    grad = torch.zeros(256, dtype=torch.bfloat16, device="cuda")
+    for elems in (1 << 62, (1 << 63) + 16, (1 << 64) - 1):
+        acc = (_native.AccumItem * 1)()
+        acc[0].grad, acc[0].grad_elems, acc[0].acc_offset, acc[0].shard_elems = grad.data_ptr(), 256, 0, elems
+        assert lib.odc_scatter_accumulate(arena.handle, acc, 1, _native.DTYPE_BF16, _native.DTYPE_F32, None) \
+            == _native.ODC_ERR_INVALID
+        assert b"exceed" in lib.odc_last_error()
+        cast = (_native.GatherCastItem * 1)()
+        cast[0].dst, cast[0].src_offset, cast[0].shard_elems = grad.data_ptr(), 0, elems
+        assert lib.odc_gather_cast(arena.handle, cast, 1, _native.DTYPE_F32, _native.DTYPE_BF16, 0, None) \
+            == _native.ODC_ERR_INVALID
+        pub = (_native.PublishItem * 1)()
+        pub[0].acc_offset, pub[0].elems, pub[0].out = 0, elems, None
+        assert lib.odc_publish(arena.handle, 0, pub, 1, _native.DTYPE_F32, _native.DTYPE_F32, 2.0, None) \
+            == _native.ODC_ERR_INVALID
     torch.cuda.synchronize()
 
 
