@@ -77,7 +77,8 @@ typedef struct odc_arena_info {
   uint64_t high_water;      /* per rank, highest offset ever handed out */
 } odc_arena_info;
 
-/* Create an arena of world_size regions of bytes_per_rank bytes each on the current device.
+/* Create an arena of world_size regions of bytes_per_rank bytes each (at most 2^60) on the
+ * current device.
  * Replaces nvshmem.core.init + NVSHMEM_SYMMETRIC_SIZE (utils.py:18-49, launch.sh:135). */
 int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flags,
                      odc_arena** out);
@@ -232,7 +233,7 @@ int odc_abi_version(void);
  *  - "rank_stagger_bytes" (extra distance between rank regions), "rank_stride_align" (rank regions
  *    start on multiples of it, default 16384 = one tile) and "alloc_align" (allocations of at
  *    least this many bytes start on multiples of it, default 16384; smaller ones on 256): read
- *    when an arena is created and rounded up to multiples of 256.
+ *    when an arena is created and rounded up to multiples of 256; at most 2^40 each.
  * Unknown names return ODC_ERR_INVALID. Results never depend on these. */
 int odc_set_option(const char* name, int64_t value);
 int odc_get_option(const char* name, int64_t* value);

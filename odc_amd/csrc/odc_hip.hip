@@ -840,6 +840,10 @@ int odc_set_option(const char* name, int64_t value) {
   if (!s) return fail(ODC_ERR_INVALID, "unknown option '%s'", name ? name : "(null)");
   const bool may_be_auto = s == &g_opt.accum_blocks_per_cu;  // -1: chosen per launch
   if (value < (may_be_auto ? -1 : 0)) return fail(ODC_ERR_INVALID, "option '%s' must be >= 0", name);
+  // the arena layout options enter address arithmetic: keep them where it cannot wrap around
+  const bool is_layout = s == &g_opt.rank_stagger_bytes || s == &g_opt.rank_stride_align || s == &g_opt.alloc_align;
+  if (is_layout && value > (int64_t(1) << 40))
+    return fail(ODC_ERR_INVALID, "option '%s' must be <= 2^40", name);
   *s = value;
   return ODC_OK;
 }
@@ -863,6 +867,7 @@ int odc_arena_create(uint32_t world_size, uint64_t bytes_per_rank, uint32_t flag
   *out = nullptr;
   if (world_size == 0) return fail(ODC_ERR_INVALID, "world_size must be >= 1");
   if (bytes_per_rank == 0) return fail(ODC_ERR_INVALID, "bytes_per_rank must be > 0");
+  if (bytes_per_rank > (uint64_t(1) << 60)) return fail(ODC_ERR_INVALID, "bytes_per_rank must be <= 2^60");
   if (flags & ~(uint32_t)(ODC_ARENA_NO_BACKING | ODC_ARENA_DRY_RUN))
     return fail(ODC_ERR_INVALID, "unknown flags 0x%x", flags);
   if (flags & ODC_ARENA_DRY_RUN) flags |= ODC_ARENA_NO_BACKING;  // a dry run never owns device memory

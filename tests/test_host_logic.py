@@ -55,6 +55,9 @@ def test_options_roundtrip_and_unknown_name():
     assert e.value.code == _native.ODC_ERR_INVALID and "no_such_knob" in e.value.message
     with pytest.raises(_native.OdcNativeError):
         _native.set_option("rank_major", -1)
+    for name in ("rank_stagger_bytes", "rank_stride_align", "alloc_align"):
+        with pytest.raises(_native.OdcNativeError):  # would wrap the arena's address arithmetic
+            _native.set_option(name, (1 << 62) + 1)
 
 
 # ---- arena bookkeeping (no device memory) ------------------------------------------------------
@@ -216,6 +219,8 @@ def test_bad_arguments_and_compute_on_unbacked_arena():
     h = ctypes.c_void_p()
     assert lib.odc_arena_create(0, 1024, 0, ctypes.byref(h)) == _native.ODC_ERR_INVALID
     assert lib.odc_arena_create(4, 0, 0, ctypes.byref(h)) == _native.ODC_ERR_INVALID
+    for absurd in ((1 << 64) - 1, (1 << 63), (1 << 60) + 1):  # sizes whose rounding or product would wrap
+        assert lib.odc_arena_create(4, absurd, _native.ODC_ARENA_NO_BACKING, ctypes.byref(h)) == _native.ODC_ERR_INVALID
     assert lib.odc_arena_create(4, 1024, 0x80, ctypes.byref(h)) == _native.ODC_ERR_INVALID
     assert lib.odc_arena_create(4, 1024, 0, None) == _native.ODC_ERR_INVALID
     assert lib.odc_arena_destroy(None) == _native.ODC_ERR_INVALID
