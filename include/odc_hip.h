@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define ODC_HIP_ABI_VERSION 2
+#define ODC_HIP_ABI_VERSION 3
 
 typedef enum odc_status {
   ODC_OK = 0,
@@ -148,6 +148,26 @@ typedef struct odc_gather_cast_item {
 
 int odc_gather_cast(odc_arena* arena, const odc_gather_cast_item* items, uint32_t n_items,
                     int src_dtype, int dst_dtype, uint32_t first_rank, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * convert — for every item and EVERY rank r, inside r's own region:
+ *     region_r[dst_offset ...][i] = cast(region_r[src_offset ...][i])      for i < elems
+ * (exact widening, round-to-nearest-even narrowing; equal dtypes make it a symmetric copy): one
+ * symmetric buffer converted into another in one launch over all ranks. It keeps a copy of the
+ * sharded parameters in the compute dtype, so that the gathers of a minibatch move 2 + 2 bytes
+ * per element instead of converting on the way: the low-precision shard that the reference's
+ * FSDP1 path copies once until flush() (odc/primitives/utils.py:103-116, odc/fsdp/fsdp1.py:239-247;
+ * there every process converts its own shard, here one launch does all W). Source and
+ * destination of an item must not overlap.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct odc_convert_item {
+  uint64_t src_offset;   /* symmetric byte offset of the source, src_dtype aligned */
+  uint64_t dst_offset;   /* symmetric byte offset of the destination, dst_dtype aligned */
+  uint64_t elems;        /* elements converted per rank */
+} odc_convert_item;
+
+int odc_convert(odc_arena* arena, const odc_convert_item* items, uint32_t n_items, int src_dtype,
+                int dst_dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * scatter-accumulate — for every item and every rank r, with g = the item's gradient viewed as

@@ -18,7 +18,10 @@ CSRC_DIR = _PKG_DIR / "csrc"
 INCLUDE_DIR = _PKG_DIR.parent / "include"
 # $ODC_HIP_LIBRARY points at a library built elsewhere (same ABI); default: the in-tree build
 LIB_PATH = Path(os.environ["ODC_HIP_LIBRARY"]) if os.environ.get("ODC_HIP_LIBRARY") else CSRC_DIR / "libodc_hip.so"
-SOURCES = [CSRC_DIR / "odc_hip.hip"]
+# host side (plain C++: arena, validation, launch planning) and device side (kernels, HIP runtime calls)
+HOST_SOURCES = [CSRC_DIR / "odc_host.cpp"]
+DEVICE_SOURCES = [CSRC_DIR / "odc_kernels.hip"]
+SOURCES = HOST_SOURCES + DEVICE_SOURCES
 # measurement-only companion: bare streaming kernels that bench.py times as the practical ceiling
 CEILING_LIB_PATH = CSRC_DIR / "libodc_ceiling.so"
 CEILING_SOURCES = [CSRC_DIR / "ceiling_kernels.hip"]
@@ -35,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "odc_arena_locate",
     "odc_gather",
     "odc_gather_cast",
+    "odc_convert",
     "odc_scatter_accumulate",
     "odc_scatter_store",
     "odc_clear",
@@ -45,7 +49,7 @@ EXPORTED_SYMBOLS = (
     "odc_get_option",
 )
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 MAX_ITEMS_PER_LAUNCH = 64
 
 ODC_OK = 0
@@ -113,6 +117,14 @@ class GatherCastItem(ctypes.Structure):
     ]
 
 
+class ConvertItem(ctypes.Structure):
+    _fields_ = [
+        ("src_offset", ctypes.c_uint64),
+        ("dst_offset", ctypes.c_uint64),
+        ("elems", ctypes.c_uint64),
+    ]
+
+
 class PublishItem(ctypes.Structure):
     _fields_ = [
         ("acc_offset", ctypes.c_uint64),
@@ -140,10 +152,19 @@ def hipcc_command(output: Path = LIB_PATH, sources=None) -> list[str]:
         "-fPIC",
         "-shared",
         f"-I{INCLUDE_DIR}",
+        f"-I{CSRC_DIR}",
         "-o",
         str(output),
-        *[str(s) for s in (SOURCES if sources is None else sources)],
+        *_with_languages(SOURCES if sources is None else sources),
     ]
+
+
+def _with_languages(sources) -> list[str]:
+    """hipcc arguments for a mixed list: .cpp files are plain C++ (host only), .hip files HIP."""
+    args = []
+    for src in sources:
+        args += ["-x", "hip" if str(src).endswith(".hip") else "c++", str(src)]
+    return args
 
 
 def _run_hipcc(cmd, verbose: bool) -> None:
@@ -210,6 +231,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.odc_arena_locate.argtypes = [vp, vp, P(u32), P(u64), P(u64)]
     lib.odc_gather.argtypes = [vp, P(GatherItem), u32, u32, vp]
     lib.odc_gather_cast.argtypes = [vp, P(GatherCastItem), u32, ci, ci, u32, vp]
+    lib.odc_convert.argtypes = [vp, P(ConvertItem), u32, ci, ci, vp]
     lib.odc_scatter_accumulate.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
     lib.odc_scatter_store.argtypes = [vp, P(AccumItem), u32, ci, ci, vp]
     lib.odc_publish.argtypes = [vp, u32, P(PublishItem), u32, ci, ci, ctypes.c_float, vp]

@@ -196,6 +196,7 @@ class ParamGroup:
                 rows = math.ceil(full.shape[0] / self.world_size)
                 chunk = full[r * rows : (r + 1) * rows].reshape(-1).to(self.dtype)
                 peers[r][self.offsets[p] : self.offsets[p] + chunk.numel()].copy_(chunk)
+        shards_may_have_changed()
 
     # -- unshard ----------------------------------------------------------------------------
     def unshard(self, fused: bool = True) -> List[torch.Tensor]:
@@ -208,6 +209,8 @@ class ParamGroup:
             padded = [torch.empty(W * n, dtype=out_dtype, device=device) for n in self.shard_numels]
             source = self.symm_buffer
             if self.compute_dtype_shards and out_dtype != self.dtype:
+                # the shards handed out by sharded_params() are views of the symmetric buffer and
+                # share its version counter: writes through them are seen without a watch list
                 source = compute_dtype_shards_of(gather, self.key, self.total_shard_numel, out_dtype)
             gather.gather_slices(padded, source, self.offsets, self.shard_numels, self.pg)
         else:
@@ -269,8 +272,9 @@ class ParamGroup:
             return None  # no microbatch touched this group in this minibatch (fsdp2.py:797-801)
         self._reduced = False
         divisor = float(self.world_size) if self.reduce_op == "avg" else 1.0
+        # the gradients are handed out as views of the slices: nothing is written between them
         (reduce_output,) = get_reduction_service().publish(
-            [id(self)], out_dtype=self.dtype, divisor=divisor
+            [id(self)], out_dtype=self.dtype, divisor=divisor, within_slices=True
         )
         rank = get_rank()
         grads = []
@@ -359,6 +363,12 @@ def replace_sharded_param_with_symm_buffer(fsdp_model) -> None:
         fp._odc_group = group
     group._odc_layout = layout
     group._odc_symm_buffer = symm_buffer
+    # a checkpoint load rewrites the shards: copies kept in the compute dtype are made anew
+    fsdp_model.register_load_state_dict_post_hook(_after_load_state_dict)
+
+
+def _after_load_state_dict(module, incompatible_keys) -> None:
+    shards_may_have_changed()
 
 
 @torch.no_grad()
@@ -398,6 +408,7 @@ def fill_peer_shards(fsdp_model, full_params) -> None:
             chunk = full[r * rows : (r + 1) * rows].reshape(-1).to(layout.dtype)
             peers[r][off : off + n].zero_()
             peers[r][off : off + chunk.numel()].copy_(chunk)
+    shards_may_have_changed()
 
 
 @torch.no_grad()
@@ -548,7 +559,7 @@ def _publish_request(fsdp_param_group):
     if ctx["all_reduce_hook"] is not None or (postdivide_factor is not None and postdivide_factor > 1):
         # two roundings (average, then post-divide) and a user hook in between
         if reduce_scatter_op == dist.ReduceOp.AVG:
-            scatter.publish([key], divisor=float(rs_group.size()))
+            scatter.publish([key], divisor=float(rs_group.size()), within_slices=ctx["all_reduce_hook"] is None)
         if ctx["all_reduce_hook"] is not None:
             ctx["all_reduce_hook"](scatter.get_accumulation(key))
         divisor = postdivide_factor if postdivide_factor is not None and postdivide_factor > 1 else 1.0
@@ -589,7 +600,8 @@ def update_gradients(fsdp_param_group) -> None:
     if request is None:
         return
     key, out_dtype, divisor, touched = request
-    (reduce_output,) = get_reduction_service().publish([key], out_dtype=out_dtype, divisor=divisor)
+    (reduce_output,) = get_reduction_service().publish([key], out_dtype=out_dtype, divisor=divisor,
+                                                       within_slices=True)
     _hand_out_gradients(fsdp_param_group, reduce_output, touched)
 
 
@@ -607,7 +619,8 @@ def update_all_gradients(fsdp_param_groups) -> None:
         key, out_dtype, divisor, touched = request
         batches.setdefault((scatter.accumulation_dtype_of(key), out_dtype, divisor), []).append((group, key, touched))
     for (_acc_dtype, out_dtype, divisor), members in batches.items():
-        outputs = scatter.publish([key for _, key, _ in members], out_dtype=out_dtype, divisor=divisor)
+        outputs = scatter.publish([key for _, key, _ in members], out_dtype=out_dtype, divisor=divisor,
+                                  within_slices=True)
         for (group, _key, touched), reduce_output in zip(members, outputs):
             with torch.cuda.nvtx.range(f"update_gradients:{group._module_fqn}"):
                 _hand_out_gradients(group, reduce_output, touched)
@@ -653,20 +666,19 @@ def pre_optimizer_step(fsdp_module):
 
 def _comm_context_lazy_init(self, device):
     """``FSDPCommContext.lazy_init`` with the all-gather and reduce-scatter streams at the default
-    priority. torch creates them at high priority so that its copy-in / copy-out kernels are not
-    delayed behind compute; the launches here gain nothing from it on MI355X (Llama example: 21.8
-    ms per microbatch with default-priority streams, 21.7 with torch's), work queued on streams
-    of different priorities is a known hazard on this platform, and it is costly: with the
-    launches on the reference's dedicated comm stream (default priority) next to torch's
-    high-priority streams the same microbatch takes 28.2 ms, with all streams at the default
-    priority 21.6. ``ODC_FSDP2_STREAM_PRIORITY=torch`` keeps torch's streams."""
+    priority, always. torch creates them at high priority so that its copy-in / copy-out kernels
+    are not delayed behind compute; the launches here gain nothing from it on MI355X (Llama
+    example: 21.8 ms per microbatch with default-priority streams, 21.7 with torch's), and work
+    queued on streams of different priorities is a hazard on this platform (it has hung) and
+    costly (with the launches on the reference's dedicated comm stream next to torch's
+    high-priority streams the same microbatch took 28.2 ms, with all streams at the default
+    priority 21.6). So there is no switch that keeps torch's priorities."""
     from torch.distributed.fsdp._fully_shard import _fsdp_param_group
 
     _fsdp_param_group.FSDPCommContext._odc_original_lazy_init(self, device)
-    if os.environ.get("ODC_FSDP2_STREAM_PRIORITY", "default") != "torch":
-        self.all_gather_copy_in_stream = self.device_handle.Stream()
-        self.all_gather_stream = self.device_handle.Stream()
-        self.reduce_scatter_stream = self.device_handle.Stream()
+    self.all_gather_copy_in_stream = self.device_handle.Stream()
+    self.all_gather_stream = self.device_handle.Stream()
+    self.reduce_scatter_stream = self.device_handle.Stream()
 
 
 def patch_fsdp2(enable_hpz: bool = False, compute_dtype_shards: Optional[bool] = None) -> None:

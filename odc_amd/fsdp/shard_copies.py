@@ -12,7 +12,9 @@ _epoch = 0  # bumped by the minibatch hooks: the sharded parameters may have cha
 
 
 def shards_may_have_changed() -> None:
-    """Every copy made so far counts as out of date (called by the minibatch hooks)."""
+    """Every copy made so far counts as out of date: the next gather converts anew. Called by the
+    minibatch hooks and by everything in this package that rewrites shards; call it after writing
+    sharded parameters in a way torch's version counters do not see."""
     global _epoch
     _epoch += 1
 
@@ -34,9 +36,14 @@ def compute_dtype_shards_of(gather_service, src_key, numel: int, dtype: torch.dt
     between them), or when torch has written to the shards since: the version counters of every rank's source
     buffer (writes through views of it: ``fill_peer_shards``, ``load_full_params``) and of the
     tensors in ``watch`` — the sharded parameters themselves, whose in-place updates as DTensors
-    (optimizers, ``load_state_dict``) bump the DTensor's counter, not its local tensor's. Code that
-    writes the shards behind torch's back, through raw pointers, must call one of the hooks
-    afterwards. The bookkeeping lives on the registry, so it ends with the arena."""
+    (optimizers, ``load_state_dict``) bump the DTensor's counter, not its local tensor's. Writes
+    that no version counter sees need ``shards_may_have_changed()`` afterwards (exported as
+    ``odc_amd.fsdp.shards_may_have_changed``): ``param.data.copy_()`` and other ``.data`` aliases
+    (a detached alias has a counter of its own), tensors built separately over the same memory
+    (``arena.view``, ``get_same_node_tensors``), raw pointers. ``fill_peer_shards``,
+    ``ParamGroup.load_full_params`` and the ``load_state_dict`` post hook of patched
+    ``fully_shard`` modules call it themselves. The bookkeeping lives on the registry, so it ends
+    with the arena."""
     registry = SymmBufferRegistry.get_instance()
     key = f"{src_key}_as_{str(dtype).rsplit('.', 1)[-1]}"
     made = registry.__dict__.setdefault("_odc_compute_dtype_shards", {})

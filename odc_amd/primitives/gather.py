@@ -13,6 +13,7 @@ import logging
 import threading
 from typing import Sequence
 
+import torch
 from torch import Tensor
 
 from odc_amd import _native
@@ -24,6 +25,7 @@ from odc_amd.primitives.utils import (
     get_world,
     group_size,
     native_dtype,
+    stream_from_handle,
 )
 
 logger = logging.getLogger(__name__)
@@ -40,6 +42,9 @@ class GatherService:
     def __init__(self):
         self.buffer_splitter = BufferSplitter()
         self._plans = threading.local()  # per host thread: plan key -> _GatherPlan
+        self._lock = threading.Lock()
+        self._conversion = None  # (stream handle, event) of the latest convert_symm_buffer
+        self._met_conversion = frozenset()  # streams ordered after it (replaced, never mutated)
 
     def gather_into_tensor(self, output_tensor: Tensor, input_tensor: Tensor, pg) -> None:
         """``output_tensor.view(W, -1)[r] = rank r's copy of input_tensor`` for every r.
@@ -132,6 +137,8 @@ class GatherService:
 
         lib = _native.load()
         with comm_stream_section("odc.gather") as comm:
+            if self._conversion is not None:
+                self._order_after_conversion(comm.cuda_stream)
             stream = ctypes.c_void_p(comm.cuda_stream)
             if plan.cast:
                 status = lib.odc_gather_cast(
@@ -178,8 +185,10 @@ class GatherService:
     def convert_symm_buffer(self, dst_key, src_key, ranks: Sequence[int] = None) -> None:
         """Rank r's symmetric buffer ``dst_key`` = rank r's ``src_key`` converted to the
         destination's dtype (round to nearest even), for every rank whose memory this process
-        holds (``ranks`` narrows it; with one process per GPU a rank converts its own shard).
-        One launch per rank, on the launch stream of the other primitives.
+        holds, in ONE launch over all W regions (``odc_convert``); ``ranks`` narrows it to some
+        ranks, one launch each (with one process per GPU a rank converts its own shard). On the
+        launch stream of the other primitives; a gather issued later on another stream first
+        waits for the conversion.
 
         It is what keeps a copy of the sharded parameters in the compute dtype: converted once
         after the optimizer step (4 + 2 bytes per element of ONE shard), so that every gather of
@@ -189,24 +198,57 @@ class GatherService:
         registry = SymmBufferRegistry.get_instance()
         world = get_world()
         src_offset, src_shape, src_dtype = registry.offsets[src_key]
-        _dst_offset, dst_shape, dst_dtype = registry.offsets[dst_key]
+        dst_offset, dst_shape, dst_dtype = registry.offsets[dst_key]
         assert tuple(src_shape) == tuple(dst_shape), f"{src_key}: {src_shape} != {dst_key}: {dst_shape}"
         numel = 1
         for d in src_shape:
             numel *= d
         if not numel:
             return
-        item = (_native.PublishItem * 1)()
-        item[0].acc_offset = src_offset
-        item[0].elems = numel
         lib = _native.load()
-        peers = registry.peer_tensors[dst_key]
         with comm_stream_section("odc.convert") as comm:
             stream = ctypes.c_void_p(comm.cuda_stream)
-            for r in range(world.world_size) if ranks is None else ranks:
-                item[0].out = peers[r].data_ptr()
+            if ranks is None:
+                item = (_native.ConvertItem * 1)()
+                item[0].src_offset, item[0].dst_offset, item[0].elems = src_offset, dst_offset, numel
                 _native.check(
-                    lib.odc_publish(
-                        world.arena.handle, r, item, 1, native_dtype(src_dtype), native_dtype(dst_dtype), 1.0, stream
-                    )
+                    lib.odc_convert(world.arena.handle, item, 1, native_dtype(src_dtype), native_dtype(dst_dtype), stream)
                 )
+            else:
+                item = (_native.PublishItem * 1)()
+                item[0].acc_offset = src_offset
+                item[0].elems = numel
+                peers = registry.peer_tensors[dst_key]
+                for r in ranks:
+                    item[0].out = peers[r].data_ptr()
+                    _native.check(
+                        lib.odc_publish(
+                            world.arena.handle, r, item, 1, native_dtype(src_dtype), native_dtype(dst_dtype), 1.0, stream
+                        )
+                    )
+            self._note_conversion(comm.cuda_stream)
+
+    def _note_conversion(self, stream_handle: int) -> None:
+        """A conversion was just launched on ``stream_handle``: gathers on other streams must
+        not read its output before it is written. Conversions are rare (one per group and
+        minibatch), so the event is recorded here, eagerly; a gather only looks at it when its
+        own stream has not met this conversion yet."""
+        if torch.cuda.is_current_stream_capturing():
+            return  # inside a graph the capture's own stream order is all there is
+        event = torch.cuda.Event()
+        event.record(stream_from_handle(stream_handle))
+        with self._lock:
+            self._conversion = (stream_handle, event)
+            self._met_conversion = {stream_handle}
+
+    def _order_after_conversion(self, stream_handle: int) -> None:
+        """Before a gather on ``stream_handle``: wait for the latest conversion if it ran on
+        another stream and this stream has not waited for it yet."""
+        if stream_handle in self._met_conversion:
+            return
+        with self._lock:
+            if self._conversion is None or stream_handle in self._met_conversion:
+                return
+            if not torch.cuda.is_current_stream_capturing():
+                stream_from_handle(stream_handle).wait_event(self._conversion[1])
+                self._met_conversion = self._met_conversion | {stream_handle}

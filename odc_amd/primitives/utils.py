@@ -243,6 +243,8 @@ def finalize_distributed():
         _world.arena.destroy()
         _world = None
     _bare_allocations.clear()
+    with _launch_lock:
+        _launch_streams.clear()  # handles of a world that is gone are not waited for
     stream = None
 
 
@@ -484,6 +486,88 @@ def get_comm_stream():
 
 
 _launch_streams = {}  # stream handle -> torch stream with launches since the last wait (None: not wrapped yet)
+_launch_lock = threading.Lock()  # launches come from several host threads (autograd's device thread)
+
+
+def stream_from_handle(handle: int):
+    """A torch stream object for a raw stream handle of the arena's device."""
+    device = get_world().arena.device
+    if handle == 0:  # the default stream: ExternalStream does not wrap a null handle
+        return torch.cuda.default_stream(device)
+    return torch.cuda.ExternalStream(handle, device=device)
+
+
+class StreamOrder:
+    """Orders launches that touch the same buffer from different streams.
+
+    In the reference every add into a rank's accumulation goes through that rank's one watcher
+    (``scatter_accumulate.py:291-310,386-392``), so clients on different streams never race on
+    it. Here a launch is a plain read-modify-write on the caller's stream; this class remembers,
+    per key, the stream of the last launch that wrote it, and when the next launch for that key
+    comes on another stream it makes the new stream wait for an event recorded on the previous
+    one. Nothing is recorded while launches stay on one stream (the steady state: one comparison
+    per call). Not thread safe on its own: the owner calls it under its lock.
+
+    Launches recorded into a HIP graph are not tracked: a graph runs on whatever stream it is
+    replayed on, which the host cannot know at capture time; ordering a replay against eager
+    launches on other streams is the caller's business, as it is for any graph."""
+
+    __slots__ = ("_base", "_last")
+
+    def __init__(self):
+        self._base = None  # the stream every key without an entry in _last was last written on
+        self._last = {}  # key -> stream handle, for the keys that differ from _base
+
+    def forget(self):
+        self._base = None
+        self._last.clear()
+
+    def before_launch(self, keys, handle: int, all_keys: bool = False, total: int = 0) -> None:
+        """Call before launching work that writes ``keys`` on stream ``handle``. ``all_keys``:
+        the launch writes every key there is; ``total``: how many keys there are (lets the
+        per-key table collapse once all of them have moved to one stream)."""
+        if not self._last:
+            if self._base == handle:
+                return
+            if self._base is None:
+                self._base = handle
+                return
+        previous = set()
+        if all_keys:
+            previous.update(self._last.values())
+            previous.add(self._base)
+            self._last.clear()
+            self._base = handle
+        else:
+            last, base = self._last, self._base
+            for key in keys:
+                previous.add(last.get(key, base))
+                if handle == base:
+                    last.pop(key, None)
+                else:
+                    last[key] = handle
+            if total and len(last) >= total and all(h == handle for h in last.values()):
+                last.clear()
+                self._base = handle
+        previous.discard(handle)
+        previous.discard(None)
+        if previous:
+            current = stream_from_handle(handle)
+            for prev in previous:
+                join_streams(current, prev)
+
+
+def join_streams(current, previous_handle: int) -> None:
+    """Make ``current`` wait for everything queued so far on the stream ``previous_handle``."""
+    event = torch.cuda.Event()
+    try:
+        event.record(stream_from_handle(previous_handle))
+    except RuntimeError:
+        # the stream no longer exists (a user stream destroyed since its launch); what it had
+        # queued may still be running, and only the device as a whole can be waited for
+        torch.cuda.synchronize(get_world().arena.device)
+        return
+    current.wait_event(event)
 
 # The two environment switches are read on every launch, so that they can be flipped at run time;
 # os.environ.get costs a microsecond per lookup (key encoding), the mapping underneath it does not.
@@ -561,12 +645,14 @@ class comm_stream_section:
             if launch_stream_policy() == "caller":
                 handle = _current_raw_stream(get_world().arena.device)
                 if handle not in _launch_streams:
-                    _launch_streams[handle] = None
+                    with _launch_lock:
+                        _launch_streams.setdefault(handle, None)
                 self.cuda_stream = handle
                 return self
             current = torch.cuda.current_stream()
             comm = get_comm_stream()
-            _launch_streams[comm.cuda_stream] = comm
+            with _launch_lock:
+                _launch_streams[comm.cuda_stream] = comm
             self.cuda_stream = comm.cuda_stream
             if current == comm:
                 return self
@@ -590,14 +676,15 @@ class comm_stream_section:
 
 def wait_for_launches() -> None:
     """Block the host until every launch issued through ``comm_stream_section`` has finished."""
-    while _launch_streams:
-        handle, s = _launch_streams.popitem()
-        if s is None:
-            if handle == 0:  # the default stream: ExternalStream does not wrap a null handle
-                s = torch.cuda.default_stream(get_world().arena.device)
-            else:
-                s = torch.cuda.ExternalStream(handle, device=get_world().arena.device)
-        s.synchronize()
+    with _launch_lock:
+        pending = list(_launch_streams.items())
+        _launch_streams.clear()
+    for handle, s in pending:
+        try:
+            (s if s is not None else stream_from_handle(handle)).synchronize()
+        except RuntimeError:
+            # a stream destroyed since its launch cannot be waited for by name
+            torch.cuda.synchronize(get_world().arena.device)
 
 
 class BufferSplitter:

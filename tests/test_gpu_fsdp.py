@@ -191,6 +191,19 @@ def test_fsdp2_group_gathers_from_shards_kept_in_the_compute_dtype(make_world):
             buf.data.mul_(-0.5)
     fsdp2.pre_minibatch_start(types.SimpleNamespace(_odc_param_groups=[kept, plain]))
     check("after the hook", 3)
+    # ... and so does the documented invalidation call on its own
+    import odc_amd.fsdp
+
+    for pgp in (kept, plain):
+        for r in range(W):
+            for shard in pgp.sharded_params(r):
+                shard.data.add_(0.25)  # .data: a detached alias with a version counter of its own
+    odc_amd.fsdp.shards_may_have_changed()
+    check("after shards_may_have_changed()", 4)
+    # loading full parameters invalidates by itself
+    for pgp in (kept, plain):
+        pgp.load_full_params([p.cuda() * 2 for p in params])
+    check("after load_full_params", 5)
     del got
     fsdp2.stop()
 

@@ -220,6 +220,96 @@ def test_gather_with_cast(make_world, src_dtype, dst_dtype, W, S):
     assert (buf[:5] == 7).all() and (buf[5 + W * S :] == 7).all()
 
 
+ALL_PAIRS = [(a, b) for a in (torch.float32, torch.bfloat16, torch.float16)
+             for b in (torch.float32, torch.bfloat16, torch.float16)]
+
+
+@pytest.mark.parametrize("src_dtype,dst_dtype", ALL_PAIRS)
+@pytest.mark.parametrize("W,n,lead", [(1, 3, 0), (8, 4096, 0), (8, 4099, 3), (12, 33_337, 1), (3, 70_001, 5), (64, 64, 0)])
+def test_convert_all_ranks_in_one_launch(make_world, src_dtype, dst_dtype, W, n, lead):
+    """odc_convert through the C ABI: every rank's slice of one symmetric buffer converted into
+    that rank's slice of another, in one launch, equals torch's CPU ``.to(dtype)`` (round to
+    nearest even) per rank; the elements around the destination slices keep their values. Equal
+    dtypes make it a symmetric copy."""
+    import ctypes
+
+    from odc_amd import _native
+    from odc_amd.primitives.utils import get_world, native_dtype
+
+    make_world(W, 4 << 20)
+    _, _, registry = services()
+    guard = 9
+    registry.allocate_symm_buffer("src", (n + lead,), src_dtype)
+    registry.allocate_symm_buffer("dst", (n + lead + 2 * guard,), dst_dtype)
+    g = torch.Generator().manual_seed(n + W)
+    shards = [(torch.randn(n + lead, generator=g) * 10.0 ** (r % 5 - 2)).to(src_dtype) for r in range(W)]
+    for peer, shard in zip(registry.peer_tensors["src"], shards):
+        peer.copy_(shard)
+    for peer in registry.peer_tensors["dst"]:
+        peer.fill_(7.0)
+    item = (_native.ConvertItem * 2)()
+    item[0].src_offset = registry.get_offset("src") + lead * src_dtype.itemsize
+    item[0].dst_offset = registry.get_offset("dst") + (guard + lead) * dst_dtype.itemsize
+    item[0].elems = n
+    item[1].elems = 0  # empty items take no part
+    _native.check(_native.load().odc_convert(
+        get_world().arena.handle, item, 2, native_dtype(src_dtype), native_dtype(dst_dtype),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    for r, peer in enumerate(registry.peer_tensors["dst"]):
+        got = peer.cpu()
+        assert_bit_equal(got[guard + lead : guard + lead + n], shards[r][lead:].to(dst_dtype), f"rank {r}")
+        assert (got[: guard + lead] == 7).all() and (got[guard + lead + n :] == 7).all(), f"rank {r}: guards"
+
+
+def test_convert_special_values_and_errors(make_world):
+    """Ties, overflow, denormals, signed zero and NaN through the one-launch conversion (fp32 ->
+    bf16), and the argument checks of odc_convert."""
+    import ctypes
+
+    from odc_amd import GatherService, _native
+    from odc_amd.primitives.utils import get_world
+
+    W = 4
+    make_world(W, 4 << 20)
+    _, _, registry = services()
+    ties = (2.0 ** torch.arange(-149, 127, dtype=torch.float64)).float() * 1.00390625
+    vals = torch.cat([ties, -ties, torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 3.4e38, -3.4e38, 1e-45, float("nan")])])
+    vals = torch.cat([vals, torch.zeros((-vals.numel()) % W)])
+    n = vals.numel() // W
+    registry.allocate_symm_buffer("m", (n,), torch.float32)
+    registry.allocate_symm_buffer("c", (n,), torch.bfloat16)
+    for peer, shard in zip(registry.peer_tensors["m"], vals.view(W, -1)):
+        peer.copy_(shard)
+    GatherService().convert_symm_buffer("c", "m")
+    torch.cuda.synchronize()
+    got = torch.cat([p.cpu() for p in registry.peer_tensors["c"]])
+    want = vals.bfloat16()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    assert_bit_equal(got[~nan], want[~nan], "ties, overflow to inf, denormals, signed zero")
+
+    lib, arena = _native.load(), get_world().arena.handle
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    src, dst = registry.get_offset("m"), registry.get_offset("c")
+
+    def status(src_offset, dst_offset, elems, sd=_native.DTYPE_F32, dd=_native.DTYPE_BF16):
+        item = (_native.ConvertItem * 1)()
+        item[0].src_offset, item[0].dst_offset, item[0].elems = src_offset, dst_offset, elems
+        return lib.odc_convert(arena, item, 1, sd, dd, stream)
+
+    assert status(src, dst, n) == _native.ODC_OK
+    assert status(src + 2, dst, n - 1) == _native.ODC_ERR_INVALID  # source not fp32 aligned
+    assert status(src, dst + 1, n - 1) == _native.ODC_ERR_INVALID  # destination not bf16 aligned
+    assert status(src, src + 4, n - 1) == _native.ODC_ERR_INVALID  # overlap
+    assert b"overlaps" in lib.odc_last_error()
+    assert status(src, dst, 1 << 62) == _native.ODC_ERR_INVALID  # byte size would wrap
+    assert status((4 << 20) - 4, dst, 2) == _native.ODC_ERR_INVALID  # leaves the rank region
+    assert status(src, dst, n, sd=7) == _native.ODC_ERR_INVALID  # unknown dtype code
+    assert lib.odc_convert(arena, None, 1, _native.DTYPE_F32, _native.DTYPE_BF16, stream) == _native.ODC_ERR_INVALID
+    torch.cuda.synchronize()
+
+
 def test_gather_with_cast_special_values(make_world):
     W = 4
     group = make_world(W, 4 << 20)

@@ -154,7 +154,7 @@ def test_slices_that_tile_the_accumulation_take_the_store_form(make_world, seed)
     red = ReductionService(accumulation_dtype=acc_dtype, lazy_clear=True)
     forms = []
     launch = red._launch
-    red._launch = lambda items, n, gc, ac, store: (forms.append(store), launch(items, n, gc, ac, store))[1]
+    red._launch = lambda keys, items, n, gc, ac, store: (forms.append(store), launch(keys, items, n, gc, ac, store))[1]
     g = torch.Generator().manual_seed(seed)
     want = [torch.zeros(total, dtype=acc_dtype) for _ in range(W)]
     order = list(range(len(sizes)))
@@ -196,7 +196,7 @@ def test_store_form_over_slices_needs_the_rest_of_the_accumulation_to_be_zero(ma
     red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=True)
     forms = []
     launch = red._launch
-    red._launch = lambda items, n, gc, ac, store: (forms.append(store), launch(items, n, gc, ac, store))[1]
+    red._launch = lambda keys, items, n, gc, ac, store: (forms.append(store), launch(keys, items, n, gc, ac, store))[1]
     g = torch.Generator().manual_seed(0)
     want = [torch.zeros(total) for _ in range(W)]
 
@@ -212,7 +212,10 @@ def test_store_form_over_slices_needs_the_rest_of_the_accumulation_to_be_zero(ma
             w.zero_()
 
     def check(msg):
-        for r, acc in enumerate(red.get_peer_accumulations("g")):
+        # the memory as it is (nothing is owed at the points checked); a public hand-out would
+        # count as a possible write between the slices, which the last part of the test covers
+        assert "g" not in red._owed_zero
+        for r, acc in enumerate(red._registry_peers("g")):
             assert_bit_equal(acc, want[r], f"{msg}: rank {r}")
 
     reduce_slices(offs, sizes)          # registers (zeroed): read-modify-write
@@ -243,6 +246,24 @@ def test_store_form_over_slices_needs_the_rest_of_the_accumulation_to_be_zero(ma
     reduce_slices(offs, sizes)          # ... and leaves data between the slices: real clear
     assert forms[7:] == [False]
     check("slices after a whole-key minibatch")
+    new_minibatch()
+    reduce_slices(offs, sizes)          # whole clear, this layout only: store
+    assert forms[8:] == [True]
+    # a live accumulation handed out with the promise to stay inside the slices keeps the store form
+    red.get_accumulation("g", within_slices=True)[offs[1] : offs[1] + 3].add_(1.0)
+    for w in want[:1]:
+        w[offs[1] : offs[1] + 3] += 1.0
+    check("written inside a slice through the live tensor")
+    new_minibatch()
+    reduce_slices(offs, sizes)
+    assert forms[9:] == [True]
+    # handed out without the promise, the holder may write between the slices: the next lazy
+    # clear is a real one, and what was written into the gap is gone after it
+    red.get_accumulation("g")[offs[0] + sizes[0] + 5] = 3.0
+    new_minibatch()
+    reduce_slices(offs, sizes)
+    assert forms[10:] == [False]
+    check("after an untracked write into a gap")
 
 
 def test_clear_stays_eager_under_graph_capture(make_world):
@@ -339,3 +360,150 @@ def test_capture_refuses_an_accumulation_that_owes_zeros(make_world):
     # the service still works eagerly afterwards
     red.scatter_accumulate("k", grad, group)
     assert_bit_equal(red.get_accumulation("k"), torch.ones(S), "store after the refused capture")
+
+
+@pytest.mark.parametrize("lazy", [True, False])
+def test_captured_minibatch_folds_the_clear_into_the_first_accumulate(make_world, lazy):
+    """One graph = one whole minibatch: clear_accumulations() + M x scatter-accumulate, captured
+    inside captured_minibatch(). The captured clear records no kernel for the keys the graph
+    accumulates into (their first accumulate is the store form) and a real clear for the key it
+    never touches. Replayed over 3 minibatches with every accumulation poisoned in between (a
+    read-modify-write of the first microbatch, or a missing clear, would show the poison), and
+    with eager work between the replays; every replay is bit-exact against the oracle."""
+    from odc_amd import ReductionService
+
+    W, M = 4, 8
+    sizes = {"a": 30_001, "b": 4096, "c": 7, "idle": 5_000}
+    group = make_world(W, 8 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=lazy)
+    g = torch.Generator().manual_seed(77)
+    keys = ["a", "b", "c"]
+    host = [[(torch.randn(W * sizes[k], generator=g) * 1e-3).bfloat16() for k in keys] for _ in range(M)]
+    for mb in host:
+        mb[0][::3] = -0.0  # a store that copied instead of adding +0 would leave -0
+    dev = [[t.cuda() for t in mb] for mb in host]
+    for k, n in sizes.items():
+        red.register(k, (n,), torch.bfloat16, torch.float32, group)
+    # one eager minibatch first (torch's capture recipe warms up eagerly)
+    red.clear_accumulations()
+    for m in range(M):
+        red.scatter_accumulate_multi(keys, dev[m], group)
+    red.sync(group)
+    for k in sizes:
+        red.get_accumulation(k)  # settles whatever a lazy clear still owes
+    torch.cuda.synchronize()
+
+    launches = []
+    real_launch = red._launch
+    real_clear = red._clear_keys
+
+    def spy_launch(keys_, items, n, grad_code, acc_code, store):
+        launches.append(("store" if store else "rmw", tuple(keys_)))
+        return real_launch(keys_, items, n, grad_code, acc_code, store)
+
+    def spy_clear(keys_):
+        keys_ = list(keys_)
+        if keys_:
+            launches.append(("clear", tuple(keys_)))
+        return real_clear(keys_)
+
+    red._launch, red._clear_keys = spy_launch, spy_clear
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), red.captured_minibatch():
+        red.clear_accumulations()
+        for m in range(M):
+            red.scatter_accumulate_multi(keys, dev[m], group)
+    red._launch, red._clear_keys = real_launch, real_clear
+    assert launches[0] == ("store", ("a", "b", "c")), launches[:2]
+    assert launches[1:M] == [("rmw", ("a", "b", "c"))] * (M - 1)
+    assert launches[M:] == [("clear", ("idle",))], "the key the graph never accumulates into is cleared by a kernel"
+
+    want = {k: [torch.zeros(sizes[k]) for _ in range(W)] for k in keys}
+    for m in range(M):
+        for k, t in zip(keys, host[m]):
+            oracle.scatter_accumulate(want[k], t)
+    for replay in range(3):
+        for k in sizes:
+            poison(red._registry_peers(k))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k in keys:
+            for r, acc in enumerate(red._registry_peers(k)):
+                assert_bit_equal(acc, want[k][r], f"replay {replay}, key {k}, rank {r}")
+        for acc in red._registry_peers("idle"):
+            assert_bit_equal(acc, torch.zeros(sizes["idle"]), f"replay {replay}: idle key cleared")
+        # the program's own eager work between replays: one more accumulate, read-modify-write
+        red.scatter_accumulate("b", dev[0][1], group)
+        torch.cuda.synchronize()
+        extra = [w.clone() for w in want["b"]]
+        oracle.scatter_accumulate(extra, host[0][1])
+        for r, acc in enumerate(red.get_peer_accumulations("b")):
+            assert_bit_equal(acc, extra[r], f"replay {replay}: eager accumulate after the replay")
+    # an eager clear outside capture still zeroes the captured keys with a kernel, lazy or not
+    red.clear_accumulations()
+    torch.cuda.synchronize()
+    for k in keys:
+        for acc in red._registry_peers(k):
+            assert_bit_equal(acc, torch.zeros(sizes[k]), "eager clear of a captured key")
+
+
+def test_captured_minibatch_settles_reads_and_gapped_slices(make_world):
+    """Inside captured_minibatch(): a key that is published before its first accumulate gets
+    its clear recorded in front of the publish; slices with gaps get a real clear (what lies
+    between them at replay time is unknown), slices that tile the accumulation take the store
+    form; and a block outside capture, or nested, is refused."""
+    from odc_amd import ReductionService
+
+    W = 4
+    group = make_world(W, 8 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="inside torch.cuda.graph"):
+        with red.captured_minibatch():
+            pass
+    sizes, gapped, tiled = [5000, 300], [0, 8192], [0, 5000]
+    g = torch.Generator().manual_seed(5)
+    host = [(torch.randn(W * n, generator=g) * 1e-3).bfloat16() for n in sizes]
+    dev = [t.cuda() for t in host]
+    red.register("read", (64,), torch.bfloat16, torch.float32, group)
+    red.scatter_accumulate_slices("gapped", dev, gapped, sizes, group, accumulation_numel=8192 + 300)
+    red.scatter_accumulate_slices("tiled", dev, tiled, sizes, group, accumulation_numel=5300)
+    red.sync(group)
+    torch.cuda.synchronize()
+    forms = []
+    real_launch, real_clear = red._launch, red._clear_keys
+    red._launch = lambda k, i, n, gc_, ac, store: (forms.append(("store" if store else "rmw", tuple(k))),
+                                                     real_launch(k, i, n, gc_, ac, store))[1]
+    red._clear_keys = lambda k: (forms.append(("clear", tuple(k))) if list(k) else None, real_clear(k))[1]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), red.captured_minibatch():
+        with pytest.raises(RuntimeError, match="do not nest"):
+            with red.captured_minibatch():
+                pass
+    graph = torch.cuda.CUDAGraph()
+    forms.clear()
+    with torch.cuda.graph(graph), red.captured_minibatch():
+        red.clear_accumulations()
+        out = red.publish(["read"], out_dtype=torch.bfloat16)[0]
+        red.scatter_accumulate_slices("gapped", dev, gapped, sizes, group)
+        red.scatter_accumulate_slices("tiled", dev, tiled, sizes, group)
+        red.scatter_accumulate_slices("tiled", dev, tiled, sizes, group)
+    red._launch, red._clear_keys = real_launch, real_clear
+    assert forms == [("clear", ("read",)), ("clear", ("gapped",)), ("rmw", ("gapped",)), ("store", ("tiled",)),
+                     ("rmw", ("tiled",))], forms
+    for replay in range(2):
+        for k in ("read", "gapped", "tiled"):
+            poison(red._registry_peers(k))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bit_equal(out, torch.zeros(64, dtype=torch.bfloat16), "published zeros")
+        for r in range(W):
+            want_g, want_t = torch.zeros(8192 + 300), torch.zeros(5300)
+            for off_g, off_t, n, t in zip(gapped, tiled, sizes, host):
+                chunk = t.view(W, n)[r].float()
+                want_g[off_g : off_g + n] += chunk
+                want_t[off_t : off_t + n] += chunk
+                want_t[off_t : off_t + n] += chunk
+            assert_bit_equal(red._registry_peers("gapped")[r], want_g, f"replay {replay} gapped rank {r}")
+            assert_bit_equal(red._registry_peers("tiled")[r], want_t, f"replay {replay} tiled rank {r}")

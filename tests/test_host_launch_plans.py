@@ -220,3 +220,51 @@ def test_many_large_items_split_when_the_tile_count_would_overflow(arena):
     _native.check(a.lib.odc_gather(a.handle, items, 3, 0, None))
     launches, tiles, _ = a.counters()
     assert (launches, tiles) == (3, 3 << 30)  # 2^30 + 2^30 would reach 2^31: one item per launch
+
+
+def test_convert_plans_one_launch_over_all_ranks(arena):
+    W = 8
+    a = arena(W)
+    C = _native.ConvertItem
+    items = (C * 3)(C(0, 1 << 24, 1_000_000), C(0, 0, 0), C(1 << 25, 1 << 26, 4096))
+    _native.check(a.lib.odc_convert(a.handle, items, 3, _native.DTYPE_F32, _native.DTYPE_BF16, None))
+    tiles = W * (math.ceil(1_000_000 / TILE_ELEMS) + 1)
+    assert a.counters() == (1, tiles, tiles)  # the empty item takes no part
+    lib = a.lib
+
+    def status(src, dst, elems, sd=_native.DTYPE_F32, dd=_native.DTYPE_BF16):
+        arr = (C * 1)(C(src, dst, elems))
+        return lib.odc_convert(a.handle, arr, 1, sd, dd, None)
+
+    assert _error(lib, status(2, 1 << 24, 64))[0] == _native.ODC_ERR_INVALID  # source not fp32 aligned
+    assert _error(lib, status(0, (1 << 24) + 1, 64))[0] == _native.ODC_ERR_INVALID  # destination not bf16 aligned
+    code, msg = _error(lib, status(0, 128, 64))  # [0, 256) read, [128, 256) written
+    assert code == _native.ODC_ERR_INVALID and "overlaps" in msg
+    assert status(0, 256, 64) == 0  # touching ranges are fine
+    code, msg = _error(lib, status(0, 1 << 24, 1 << 62))  # elems * 4 would wrap around
+    assert code == _native.ODC_ERR_INVALID and "exceed" in msg
+    assert _error(lib, status(0, a.info.bytes_per_rank - 64, 64))[0] == _native.ODC_ERR_INVALID  # destination leaves the region
+    assert _error(lib, status(0, 1 << 24, 64, sd=9))[0] == _native.ODC_ERR_INVALID
+    assert lib.odc_convert(a.handle, None, 2, _native.DTYPE_F32, _native.DTYPE_BF16, None) == _native.ODC_ERR_INVALID
+    # equal dtypes: a symmetric copy
+    assert status(0, 1 << 24, 4096, sd=_native.DTYPE_BF16, dd=_native.DTYPE_BF16) == 0
+
+
+def test_arena_size_plus_alignment_slack_cannot_wrap():
+    """world * rank_stride can fit 64 bits while the allocation, which is one stride alignment
+    larger so that rank 0 can start on a multiple of it, does not: 17 regions of 986 895 * 2^40
+    bytes are 2^64 - 2^40 bytes. Such an arena is refused, with or without backing."""
+    lib = _native.load()
+    handle = ctypes.c_void_p()
+    _native.set_option("rank_stride_align", 1 << 40)
+    try:
+        stride = 986_895 << 40
+        assert 17 * stride == (1 << 64) - (1 << 40)
+        for flags in (_native.ODC_ARENA_DRY_RUN, _native.ODC_ARENA_NO_BACKING):
+            assert lib.odc_arena_create(17, stride, flags, ctypes.byref(handle)) == _native.ODC_ERR_INVALID
+            assert "overflows" in lib.odc_last_error().decode() and not handle.value
+        # one region fewer fits
+        _native.check(lib.odc_arena_create(16, stride, _native.ODC_ARENA_NO_BACKING, ctypes.byref(handle)))
+        _native.check(lib.odc_arena_destroy(handle))
+    finally:
+        _native.set_option("rank_stride_align", 16384)

@@ -396,3 +396,16 @@ def test_fsdp2_accumulation_slices_start_on_tiles():
     assert tile_aligned_offsets([3, 5, 7]) == ([0, 3, 8], 15)
     assert tile_aligned_offsets([]) == ([], 0)
     assert tile_aligned_offsets([4096, 4096]) == ([0, 4096], 8192)
+
+
+def test_under_the_sanitizer_run_the_sanitized_library_is_the_one_loaded():
+    """tests/test_host_sanitizers.py runs this file against a g++ AddressSanitizer + UBSan build of
+    the host side; there, prove that this build (and the sanitizer runtime) is what is mapped."""
+    import os
+
+    if os.environ.get("ODC_EXPECT_SANITIZED") != "1":
+        pytest.skip("only meaningful inside the sanitizer run")
+    _native.load()
+    maps = open("/proc/self/maps").read()
+    assert os.environ["ODC_HIP_LIBRARY"] in maps and "libasan" in maps
+    assert str(_native.CSRC_DIR / "libodc_hip.so") not in maps

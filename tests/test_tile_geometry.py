@@ -37,10 +37,14 @@ def test_every_unit_is_owned_by_exactly_one_tile_role(checker, seed):
 
 
 def test_the_library_is_built_from_the_checked_header():
-    """The kernels must take their geometry from odc_tiles.h, not from a private copy."""
-    text = (ROOT / "odc_amd" / "csrc" / "odc_hip.hip").read_text()
-    assert '#include "odc_tiles.h"' in text
-    for name in ("cursor_seek(", "cursor_enter(", "cursor_coord(", "seg_shape(", "tile_work(", "fill_tile_table("):
-        assert name in text, name
+    """The kernels and the launch planning must take their geometry from odc_tiles.h, not from a
+    private copy."""
+    csrc = ROOT / "odc_amd" / "csrc"
+    device, host = (csrc / "odc_kernels.hip").read_text(), (csrc / "odc_host.cpp").read_text()
+    for text in (device, host):
+        assert '#include "odc_tiles.h"' in text
+    for name in ("cursor_seek(", "cursor_enter(", "cursor_coord(", "seg_shape(", "tile_work("):
+        assert name in device, name
+    assert "fill_tile_table(" in host
     for private in ("struct TileTable", "struct SegShape", "TileCoord locate_tile"):
-        assert private not in text, f"{private} is defined in odc_hip.hip again"
+        assert private not in device + host, f"{private} is defined outside odc_tiles.h again"
