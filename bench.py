@@ -20,12 +20,14 @@ streaming kernels of libodc_ceiling.so reach on flat arrays of the same sizes in
 profiles/traffic.json; null when a launch knob is overridden), `host_us_per_call` (host time of one
 call of each service entry point on the 9-parameter layer), the clear, the CPU oracle timed on
 the host cores (`cpu_baseline`), the parity verdict against that oracle, and `other_clear_mode`:
-the same steps launched eagerly with lazy clears, where no clear kernel runs and the first
-scatter-accumulate of a minibatch stores instead (6N bytes, counted as such).
+the same minibatches with lazy clears, replayed from a graph captured inside
+`ReductionService.captured_minibatch()`: no clear kernel runs and the first scatter-accumulate of
+a minibatch stores instead (6N bytes, counted as such), checked against the oracle as well.
 
 Other workloads (not the headline): `--workload uneven --world-size 12` (40 uneven, zero-padded
-flat parameters), `--workload model` (the whole 8.03 G-parameter model), `--layout flat`,
-`--world-size 64`.
+flat parameters), `--workload model` (the whole 8.03 G-parameter model, swept unit by unit: sampled
+units against the oracle, per-unit-shape roofline figures, a CPU baseline extrapolated from the
+embedding and one layer), `--layout flat`, `--world-size 64`.
 """
 
 from __future__ import annotations
@@ -75,22 +77,25 @@ def parse_args():
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--lazy-clear", action="store_true",
                     help="lazy clears for the headline: no clear kernel, the first scatter-accumulate of a "
-                         "minibatch stores instead (6N bytes); implies --no-graph (the choice between store "
-                         "and read-modify-write is host state). The default keeps the reference's eager "
-                         "clears, so that every timed scatter-accumulate is the 10N read-modify-write")
+                         "minibatch stores instead (6N bytes); graphs are then captured inside "
+                         "captured_minibatch(). The default keeps the reference's eager clears, so that every "
+                         "timed scatter-accumulate is the 10N read-modify-write")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="libodc_hip launch knob, e.g. accum_blocks_per_cu=4")
-    args = ap.parse_args()
-    if args.lazy_clear:
-        args.no_graph = True
-    return args
+    return ap.parse_args()
 
 
 def model_sweep(args):
-    """Full Llama-3-8B: per step (= microbatch), gather the 34 FSDP units in forward order, then
-    scatter-accumulate them in reverse order; every 8th step first clears all accumulations."""
+    """Full Llama-3-8B (cfg 5): per step (= microbatch), gather the 34 FSDP units in forward order,
+    then scatter-accumulate them in reverse order; every 8th step first clears all accumulations.
+
+    Parity: one eager minibatch, then the sampled units (embedding, two layers, head) against the
+    CPU oracle, gather and all W accumulations, bit for bit. CPU baseline: the oracle timed on the
+    embedding and one layer (a ninth of the model's bytes) and extrapolated to the sweep. Roofline:
+    an eager event phase with one HIP event after every launch, reported for the scatter-accumulate
+    over the whole sweep and per unit shape."""
     import torch
 
     import odc_amd
@@ -128,19 +133,101 @@ def model_sweep(args):
         plan.append((keys, [registry.get_symm_buffer(k) for k in keys], *by_shape[sig]))
     torch.cuda.synchronize()
     comm = get_comm_stream()
+    shape_of = ["embedding"] + ["layer"] * (len(units) - 2) + ["head"]
+    unit_elems = [sum(numel(s) for _, s in unit) for _, unit in units]
+    marks = []
 
-    def step(i):
+    def mark(label):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(comm)
+        marks.append((label, ev))
+
+    def step(i, record=False):
         if i % MICROBATCHES == 0:
             reduction.clear_accumulations()
-        for keys, locals_, outs, grads in plan:
+            if record and not reduction.lazy_clear:
+                mark(("clear", "all"))
+        for u, (keys, locals_, outs, grads) in enumerate(plan):
             gather.gather_into_tensors(outs, locals_, group)
-        for keys, locals_, outs, grads in reversed(plan):
+            if record:
+                mark(("gather", shape_of[u]))
+        store = reduction.lazy_clear and i % MICROBATCHES == 0
+        for u in reversed(range(len(plan))):
+            keys, locals_, outs, grads = plan[u]
             reduction.scatter_accumulate_multi(keys, grads[i % 2], group)
+            if record:
+                mark(("store" if store else "accum", shape_of[u]))
 
+    # ---- parity + CPU baseline on sampled units -------------------------------------------------
+    parity = cpu_baseline = None
+    if not args.no_verify or not args.no_cpu_baseline:
+        from oracle import odc_oracle as oracle
+
+        with torch.cuda.stream(comm):
+            for i in range(MICROBATCHES):
+                step(i)
+        reduction.sync(group)
+        sampled = [0, 1, len(units) // 2, len(units) - 1]  # embedding, two layers, norm + lm_head
+        timed_units = {0, 1}  # the CPU baseline's sample: the embedding and one layer
+        parity = True
+        cpu_s = cpu_bytes = 0.0
+        cpu_passes = 0
+        for u in sampled:
+            keys, locals_, outs, grads = plan[u]
+            host_shards = [[peer.cpu() for peer in registry.peer_tensors[k]] for k in keys]
+            host_grads = [[g.cpu() for g in mb] for mb in grads]
+            host_outs = [torch.empty(o.numel(), dtype=torch.bfloat16) for o in outs]
+            host_accs = [[torch.zeros(o.numel() // W) for _ in range(W)] for o in outs]
+
+            def cpu_minibatch():
+                for m in range(MICROBATCHES):
+                    for o, sh in zip(host_outs, host_shards):
+                        oracle.gather_into_tensor(o, sh)
+                    for accs, g in zip(host_accs, host_grads[m % 2]):
+                        oracle.scatter_accumulate(accs, g)
+
+            t0 = time.perf_counter()
+            cpu_minibatch()  # the values the GPU is checked against
+            first_s = time.perf_counter() - t0
+            if not args.no_verify:
+                with torch.cuda.stream(comm):
+                    gather.gather_into_tensors(outs, locals_, group)  # the buffers are shared by shape: gather again
+                torch.cuda.synchronize()
+                for o, ho in zip(outs, host_outs):
+                    parity &= torch.equal(o.cpu().view(torch.int16), ho.view(torch.int16))
+                for key, accs in zip(keys, host_accs):
+                    for r, acc in enumerate(reduction.get_peer_accumulations(key)):
+                        parity &= torch.equal(acc.cpu().view(torch.int32), accs[r].view(torch.int32))
+            if u in timed_units and not args.no_cpu_baseline:
+                budget = args.cpu_seconds * unit_elems[u] / sum(unit_elems[t] for t in timed_units)
+                spent, passes = first_s, 1
+                while spent < budget:
+                    t0 = time.perf_counter()
+                    cpu_minibatch()
+                    spent += time.perf_counter() - t0
+                    passes += 1
+                cpu_s += spent
+                cpu_bytes += passes * MICROBATCHES * 14 * unit_elems[u]
+                cpu_passes += passes
+            del host_shards, host_grads, host_outs, host_accs
+        parity = bool(parity) if not args.no_verify else None
+        if parity is False:
+            print("PARITY FAILURE: GPU results differ from the CPU oracle on a sampled unit", file=sys.stderr)
+        if not args.no_cpu_baseline:
+            rate = cpu_bytes / cpu_s / 1e9
+            cpu_baseline = {
+                "value": round(rate, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{cpu_passes} minibatches of {MICROBATCHES} microbatches over the embedding and one decoder "
+                          f"layer ({sum(unit_elems[t] for t in timed_units)} of {N} elements) through the torch CPU "
+                          f"oracle, {cpu_s:.1f} s; EXTRAPOLATED to the sweep at that rate: "
+                          f"{14 * N / rate / 1e9:.2f} s per microbatch",
+            }
+
+    # ---- headline: exactly --steps steps, eager launches ------------------------------------------
     gc.collect()
     gc.disable()
     with torch.cuda.stream(comm):
-        for i in range(args.warmup):
+        for i in range(-(-args.warmup // MICROBATCHES) * MICROBATCHES):
             step(i)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -151,7 +238,73 @@ def model_sweep(args):
         e1.record(comm)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
+        # ---- eager event phase: one event after every launch --------------------------------------
+        mark(("start", ""))
+        for i in range(MICROBATCHES if args.event_steps > 0 else 0):  # one minibatch: 544 launches
+            step(i, record=True)
+        torch.cuda.synchronize()
     gc.enable()
+    if args.calibrate:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
+
+    durations = {}
+    for (_, before), (label, after) in zip(marks, marks[1:]):
+        durations.setdefault(label, []).append(before.elapsed_time(after))
+    shape_elems = {"embedding": unit_elems[0], "layer": unit_elems[1], "head": unit_elems[-1]}
+    traffic = load_traffic(args, W)
+
+    def kernel_figures(kind, bytes_per_elem):
+        """Per unit shape and over the whole sweep: mean launch time, GB/s, fraction of peak."""
+        per_shape, total_bytes, total_ms = {}, 0.0, 0.0
+        for shape, elems in shape_elems.items():
+            times = durations.get((kind, shape))
+            if not times:
+                continue
+            ms = statistics.fmean(times)
+            gbps = bytes_per_elem * elems / (ms * 1e-3) / 1e9
+            per_shape[shape] = {"elements": elems, "avg_launch_ms": round(ms, 5), "launches_timed": len(times),
+                                "GB/s": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+            total_bytes += bytes_per_elem * elems * len(times)
+            total_ms += sum(times)
+        if not per_shape:
+            return None, None, None
+        return per_shape, total_bytes, total_ms
+
+    roofline = roofline_gather = None
+    accum_shapes, accum_bytes, accum_ms = kernel_figures("accum", 10)
+    if accum_shapes:
+        launches = sum(v["launches_timed"] for v in accum_shapes.values())
+        gbps = accum_bytes / (accum_ms * 1e-3) / 1e9
+        entry = traffic.get("accum:embedding", (None, None))
+        roofline = {
+            "kernel": "accum_kernel<bf16,f32> (scatter-accumulate), all launches of the sweep",
+            "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes": round(accum_bytes / launches), "avg_launch_ms": round(accum_ms / launches, 5),
+            "launches_timed": launches,
+            "traffic": entry[0], "traffic_source": entry[1],
+            "traffic_launch": "the embedding-sized launch (algorithmic bytes "
+                              f"{10 * shape_elems['embedding']})" if entry[0] else None,
+            "by_unit_shape": accum_shapes,
+        }
+    gather_shapes, gather_bytes, gather_ms = kernel_figures("gather", 4)
+    if gather_shapes:
+        launches = sum(v["launches_timed"] for v in gather_shapes.values())
+        gbps = gather_bytes / (gather_ms * 1e-3) / 1e9
+        entry = traffic.get("gather:embedding", (None, None))
+        roofline_gather = {
+            "kernel": "gather_kernel, all launches of the sweep", "bound": "hbm", "achieved": round(gbps, 1),
+            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes": round(gather_bytes / launches), "avg_launch_ms": round(gather_ms / launches, 5),
+            "launches_timed": launches, "traffic": entry[0], "traffic_source": entry[1],
+            "by_unit_shape": gather_shapes,
+        }
+    store_shapes, _, _ = kernel_figures("store", 6)
+    clear_ms = statistics.fmean(durations[("clear", "all")]) if durations.get(("clear", "all")) else None
+
     stores = len(range(0, args.steps, MICROBATCHES)) if args.lazy_clear else 0  # 6N instead of 10N
     step_bytes = (args.steps * 14 * N - stores * 4 * N) / args.steps
     value = args.steps * step_bytes / elapsed / 1e9
@@ -162,16 +315,23 @@ def model_sweep(args):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"cfg5: full Llama-3-8B ({N} bf16 params, {len(units)} units, {2 * len(units)} "
                                f"launches per step), W={W} virtual shards", "world_size": W, "elements": N,
-                   "bytes_per_step": round(step_bytes),
+                   "bytes_per_step": round(step_bytes), "launch": "eager",
                    "clear": "lazy (store on the first microbatch)" if args.lazy_clear else "eager"},
         "minibatch_ms": round(elapsed / args.steps * MICROBATCHES * 1e3, 3),
         "frac_of_peak": round(value / HBM_PEAK_GBPS, 4),
         "gpu_ms_per_step": round(e0.elapsed_time(e1) / args.steps, 3),
-        "roofline": None, "cpu_baseline": None, "parity_vs_oracle": None,
+        "roofline": roofline, "roofline_gather": roofline_gather,
+        "store": store_shapes,
+        "clear": {"avg_launch_ms": round(clear_ms, 4), "GB/s": round(4 * N / (clear_ms * 1e-3) / 1e9, 1)} if clear_ms else None,
+        "cpu_baseline": cpu_baseline, "parity_vs_oracle": parity,
+        "parity_sample": "units 0 (embedding), 1 and 17 (decoder layers), 33 (final norm + lm_head): gathered "
+                         "parameters and all W accumulations after one minibatch, bit for bit",
     }))
     torch.cuda.synchronize()
     registry.finalize()
     odc_amd.finalize_distributed()
+    if parity is False:
+        sys.exit(1)
 
 
 def load_traffic(args, W):
@@ -186,8 +346,10 @@ def load_traffic(args, W):
     out = {}
     for e in table.get("entries", []):
         if (e.get("workload"), e.get("layout"), e.get("world_size")) == (args.workload, args.layout, W):
-            out[e["kernel"]] = (e["hbm_bytes_per_launch"],
-                                f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {e['profile']} (not measured by this run)")
+            # the model sweep launches one kernel at several sizes: its entries name the unit shape
+            name = e["kernel"] + (":" + e["unit_shape"] if e.get("unit_shape") else "")
+            out[name] = (e["hbm_bytes_per_launch"],
+                         f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {e['profile']} (not measured by this run)")
     return out
 
 
@@ -493,18 +655,28 @@ def main():
     gc.disable()
     full, rest = divmod(args.steps, MICROBATCHES)
     graph_mb = graph_rest = None
-    if not args.no_graph:
-        # one graph per whole minibatch, one for the steps left over (both start with the clear)
-        torch.cuda.synchronize()
-        graph_mb = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph_mb):
-            for i in range(MICROBATCHES):
-                step(i)
-        if rest:
-            graph_rest = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph_rest):
-                for i in range(rest):
+
+    def capture_steps(n):
+        """One graph holding the first n steps of a minibatch (it starts with the clear). With lazy
+        clears the capture runs inside captured_minibatch(): the captured clear records nothing and
+        the first scatter-accumulate is recorded in the store form."""
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            if reduction.lazy_clear:
+                with reduction.captured_minibatch():
+                    for i in range(n):
+                        step(i)
+            else:
+                for i in range(n):
                     step(i)
+        return graph
+
+    if not args.no_graph:
+        # one graph per whole minibatch, one for the steps left over
+        torch.cuda.synchronize()
+        graph_mb = capture_steps(MICROBATCHES)
+        if rest:
+            graph_rest = capture_steps(rest)
         torch.cuda.synchronize()
 
     def run_steps(n_full, n_rest):
@@ -536,6 +708,8 @@ def main():
             parity = bool(parity and graph_parity)
 
         # ---- eager event phase: per-kernel durations ------------------------------------------
+        graph_mb = graph_rest = None  # destroyed: nothing replays into the accumulations any more,
+        reduction.forget_captured_graphs()  # so lazy clears may skip the clear kernel again
         for i in range(MICROBATCHES):
             step(i)
         torch.cuda.synchronize()
@@ -544,26 +718,51 @@ def main():
             step(i, record=True)
         torch.cuda.synchronize()
 
-        # the same steps once more, eagerly, in the other clear mode (no events): a secondary figure
+        # the same steps once more in the other clear mode (no events): a secondary figure,
+        # replayed from one graph per minibatch like the headline (capture_steps)
         other = None
         if args.steps >= MICROBATCHES:
-            graph_mb = graph_rest = None  # destroyed: nothing replays into the accumulations any more
-            reduction.forget_captured_graphs()
             reduction.lazy_clear = not args.lazy_clear
             for i in range(MICROBATCHES):
                 step(i)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            for i in range(args.steps):
-                step(i)
-            torch.cuda.synchronize()
-            other_elapsed = time.perf_counter() - t1
-            stores = len(range(0, args.steps, MICROBATCHES)) if reduction.lazy_clear else 0
-            other_bytes = 14 * N * args.steps - 4 * N * stores
+            reduction.sync(group)
+            other_parity = None
+            if args.no_graph:
+                t1 = time.perf_counter()
+                for i in range(args.steps):
+                    step(i)
+                torch.cuda.synchronize()
+                other_elapsed = time.perf_counter() - t1
+                other_steps = args.steps
+            else:
+                other_graph = capture_steps(MICROBATCHES)
+                other_graph.replay()
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                for _ in range(max(full, 1)):
+                    other_graph.replay()
+                torch.cuda.synchronize()
+                other_elapsed = time.perf_counter() - t1
+                other_steps = max(full, 1) * MICROBATCHES
+                if not args.no_verify and check_accs is not None:
+                    other_parity = check_against(check_outs, check_accs)
+                    if not other_parity:
+                        print("PARITY FAILURE: the captured minibatch with the clear folded into a store differs "
+                              "from the CPU oracle", file=sys.stderr)
+                    parity = bool(parity and other_parity)
+                del other_graph
+                reduction.forget_captured_graphs()
+            stores = len(range(0, other_steps, MICROBATCHES)) if reduction.lazy_clear else 0
+            other_bytes = 14 * N * other_steps - 4 * N * stores
             other = {"clear": "lazy (store on the first microbatch)" if reduction.lazy_clear else "eager",
-                     "launch": "eager", "value": round(other_bytes / other_elapsed / 1e9, 1), "unit": "GB/s",
-                     "bytes_per_step": round(other_bytes / args.steps),
-                     "minibatch_ms": round(other_elapsed / args.steps * MICROBATCHES * 1e3, 4)}
+                     "launch": "eager" if args.no_graph else
+                               f"HIP graph replay ({max(full, 1)} x one minibatch of {MICROBATCHES} steps"
+                               + (", clear folded into the first scatter-accumulate)" if reduction.lazy_clear else ")"),
+                     "value": round(other_bytes / other_elapsed / 1e9, 1), "unit": "GB/s",
+                     "frac_of_peak": round(other_bytes / other_elapsed / 1e9 / HBM_PEAK_GBPS, 4),
+                     "bytes_per_step": round(other_bytes / other_steps), "steps": other_steps,
+                     "minibatch_ms": round(other_elapsed / other_steps * MICROBATCHES * 1e3, 4),
+                     "parity_vs_oracle": other_parity}
             reduction.lazy_clear = args.lazy_clear
             reduction.clear_accumulations()
             reduction.sync(group)
