@@ -82,6 +82,10 @@ def parse_args():
                          "timed scatter-accumulate is the 10N read-modify-write")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
+    ap.add_argument("--probe", choices=["alignment", "overlap"],
+                    help="instead of the benchmark, print one of two measurement tables: alignment (what a buffer "
+                         "shifted off the 16 KiB tile grid costs the scatter-accumulate and the gather), overlap (how "
+                         "much of a gather / scatter-accumulate hides behind a co-running GEMM, by launch shape)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="libodc_hip launch knob, e.g. accum_blocks_per_cu=4")
     return ap.parse_args()
@@ -506,12 +510,172 @@ def measure_host_overhead(torch, odc_amd, comm, group, gather, reduction, regist
     return result
 
 
+def probe_alignment(args, repeats=9, launches=20):
+    """`--probe alignment`: what a misaligned buffer costs the streaming kernels. One
+    scatter-accumulate (bf16 into fp32, read-modify-write) and one gather of a buffer too large for
+    the last-level cache, with the accumulation slice, the gradient, the shard slice and the output
+    each shifted by 0 ... 16 KiB. (On MI355X the read-modify-write loses up to 5.5 % when its tiles
+    start 8 KiB past a 16 KiB boundary of the ACCUMULATION and nothing when the gradient is shifted,
+    the gather about 1 % per shifted side: why the arena and the FSDP2 group layout start buffers
+    and slices on tile boundaries.) Median of `repeats` intervals of `launches` launches."""
+    import torch
+
+    import odc_amd as odc
+
+    W = args.world_size
+    torch.cuda.set_device(0)
+    n_acc = 6656 * 4096  # elements per rank of the accumulate: 109 MB of fp32 per rank
+    n_gat = 2 * n_acc    # bf16 elements per rank of the gather: 109 MB per rank
+    slack = 16384
+    group = odc.init_nvshmem(world_size=W, symmetric_size=(n_acc + slack) * 4 + (n_gat + slack) * 2 + (8 << 20))
+    registry = odc.SymmBufferRegistry.get_instance()
+    gather, reduction = odc.GatherService(), odc.ReductionService(accumulation_dtype=torch.float32)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(launches):
+                fn()
+            e1.record()
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) / launches)
+        return statistics.median(samples)
+
+    shifts = (0, 2048, 4096, 8192, 12288, 16384)
+    outside = torch.empty(W * n_gat * 2 + (1 << 20), dtype=torch.uint8, device="cuda")  # gradient, then output
+    outside.view(torch.bfloat16).normal_(0, 1e-3)
+    reduction.register("acc", (n_acc + slack,), torch.bfloat16, torch.float32, group)
+    print(f"scatter-accumulate, {W} x {n_acc} elements, GB/s by byte shift of the slice in the accumulation (rows) "
+          f"and of the gradient (columns)")
+    print(f"{'':>8s}" + "".join(f"{g:>8d}" for g in shifts))
+    for a in shifts:
+        row = []
+        for g in shifts:
+            grad = outside[g:g + W * n_acc * 2].view(torch.bfloat16)
+            ms = timed(lambda: reduction.scatter_accumulate_slices("acc", [grad], [a // 4], [n_acc], group))
+            row.append(10 * W * n_acc / ms / 1e6)
+        print(f"{a:>8d}" + "".join(f"{x:8.0f}" for x in row), flush=True)
+    shards = registry.allocate_symm_buffer("shards", (n_gat + slack,), torch.bfloat16)
+    print(f"gather, {W} x {n_gat} bf16 elements, GB/s by byte shift of the shard slice (rows) and of the output (columns)")
+    print(f"{'':>8s}" + "".join(f"{d:>8d}" for d in shifts))
+    for sh in shifts:
+        row = []
+        for d in shifts:
+            out = outside[d:d + W * n_gat * 2].view(torch.bfloat16)
+            ms = timed(lambda: gather.gather_slices([out], shards, [sh // 2], [n_gat], group))
+            row.append(4 * W * n_gat / ms / 1e6)
+        print(f"{sh:>8d}" + "".join(f"{x:8.0f}" for x in row), flush=True)
+    torch.cuda.synchronize()
+    registry.finalize()
+    odc.finalize_distributed()
+
+
+def probe_overlap(args, gemm=8192, launches=8, repeats=5):
+    """`--probe overlap`: how much of a gather / scatter-accumulate hides behind compute on ONE
+    GPU. The reference hops to a side stream so that its data movement overlaps the model's compute
+    (odc/primitives/gather.py:114-176, utils.py:205-209); there the movement crosses NVLink, here it
+    is a streaming kernel that competes with the compute kernels for the same CUs and the same HBM.
+    A chain of bf16 GEMMs (compute bound) on one stream, the layer's gather or scatter-accumulate
+    launches on another, alone and together, by launch shape:
+        hidden = (t_gemm + t_path - t_both) / t_path      1 = free, 0 = fully serialised"""
+    import torch
+
+    import odc_amd as odc
+    from odc_amd import _native
+    from odc_amd.workloads import llama3_8b_layer_shapes, numel
+
+    W = args.world_size
+    torch.cuda.set_device(0)
+    numels = [numel(s) for _, s in llama3_8b_layer_shapes()]
+    N = sum(numels)
+    group = odc.init_nvshmem(world_size=W, symmetric_size=sum((n // W) * 6 + 512 for n in numels) + (1 << 20))
+    registry = odc.SymmBufferRegistry.get_instance()
+    gather, reduction = odc.GatherService(), odc.ReductionService(accumulation_dtype=torch.float32)
+    keys = list(range(len(numels)))
+    shards = [registry.allocate_symm_buffer(k, (n // W,), torch.bfloat16) for k, n in zip(keys, numels)]
+    for k in keys:
+        for peer in registry.peer_tensors[k]:
+            peer.normal_(0, 0.02)
+    outs = [torch.empty(n, dtype=torch.bfloat16, device="cuda") for n in numels]
+    grads = [torch.empty(n, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3) for n in numels]
+    for k, n in zip(keys, numels):
+        reduction.register(k, (n // W,), torch.bfloat16, torch.float32, group)
+    a = torch.randn(gemm, gemm, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(gemm, gemm, device="cuda", dtype=torch.bfloat16)
+    c = torch.empty_like(a)
+    compute, side = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def run_gather():
+        for _ in range(launches):
+            gather.gather_into_tensors(outs, shards, group)
+
+    def run_accum():
+        for _ in range(launches):
+            reduction.scatter_accumulate_multi(keys, grads, group)
+
+    def one(fn_side, n_gemm):
+        """Wall time of n_gemm GEMMs on `compute` and fn_side on `side`, started together."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        if n_gemm:
+            with torch.cuda.stream(compute):
+                for _ in range(n_gemm):
+                    torch.matmul(a, b, out=c)
+        if fn_side is not None:
+            with torch.cuda.stream(side):
+                fn_side()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    def best(fn_side, n_gemm):
+        one(fn_side, n_gemm)
+        return min(one(fn_side, n_gemm) for _ in range(repeats))
+
+    t_gemm1 = best(None, 4) / 4
+    print(f"bf16 GEMM {gemm}^3: {t_gemm1 * 1e3:.3f} ms = {2 * gemm ** 3 / t_gemm1 / 1e12:.0f} TFLOP/s; "
+          f"layer of {N} elements, W={W}, {launches} launches per measurement")
+    print(f"{'path kernel, launch shape':62s} {'alone ms':>9s} {'gemm ms':>8s} {'both ms':>8s} {'hidden':>7s}")
+
+    def report(label, fn_side, options):
+        for name, value in options.items():
+            _native.set_option(name, value)
+        t_path = best(fn_side, 0)
+        n_gemm = max(1, round(t_path / t_gemm1))  # compute of about the same length
+        t_gemm = best(None, n_gemm)
+        t_both = best(fn_side, n_gemm)
+        hidden = (t_gemm + t_path - t_both) / t_path
+        print(f"{label:62s} {t_path * 1e3:9.3f} {t_gemm * 1e3:8.3f} {t_both * 1e3:8.3f} {hidden:7.2f}")
+
+    report("gather, one 512-thread workgroup per tile (default: 4 fit a CU)", run_gather, {"gather_resident_cap": 0})
+    report("gather, one workgroup per tile, <= 2 resident per CU (LDS claim)", run_gather, {"gather_resident_cap": 2})
+    report("gather, 1 persistent workgroup per CU", run_gather, {"gather_blocks_per_cu": 1})
+    _native.set_option("gather_blocks_per_cu", 0)
+    _native.set_option("gather_resident_cap", 0)
+    report("scatter-accumulate, one workgroup per tile, no cap (default)", run_accum,
+           {"accum_blocks_per_cu": 0, "accum_resident_cap": 0})
+    report("scatter-accumulate, one workgroup per tile, <= 4 resident per CU", run_accum,
+           {"accum_blocks_per_cu": 0, "accum_resident_cap": 4})
+    report("scatter-accumulate, 1 persistent workgroup per CU", run_accum, {"accum_blocks_per_cu": 1})
+    _native.set_option("accum_blocks_per_cu", -1)
+    _native.set_option("accum_resident_cap", 0)
+    torch.cuda.synchronize()
+    registry.finalize()
+    odc.finalize_distributed()
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: W virtual ranks share one MI355X and nothing here uses a "
               "second GPU. Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.probe:
+        return (probe_alignment if args.probe == "alignment" else probe_overlap)(args)
     if args.workload == "model":
         return model_sweep(args)
 

@@ -681,6 +681,49 @@ def _comm_context_lazy_init(self, device):
     self.reduce_scatter_stream = self.device_handle.Stream()
 
 
+_RECORD_FUNCTION_HOMES = ("torch.distributed.fsdp._fully_shard._fsdp_param_group", "torch.profiler",
+                          "torch.autograd.profiler")
+_original_record_functions = {}
+
+
+def _forward_record_function_to_markers() -> None:
+    """torch's ``record_function`` ranges (FSDP brackets unshard, reshard, the hooks and the
+    reductions with them) also as marker ranges, so that a ``rocprofv3 --marker-trace`` timeline
+    shows them around the primitive launches: the reference's ``nvtx_record_function``, installed
+    in the same three places (fsdp2.py:54-61, 1131-1133). Here only under ``ODC_TRACE=1``, the
+    switch of the primitives' own marker ranges; ``unpatch_fsdp2`` puts torch's class back."""
+    import importlib
+
+    from torch.autograd.profiler import record_function
+
+    if _original_record_functions:
+        return
+
+    class marker_record_function(record_function):
+        def __enter__(self):
+            torch.cuda.nvtx.range_push(self.name)
+            return super().__enter__()
+
+        def __exit__(self, exc_type, exc_value, traceback):
+            try:
+                return super().__exit__(exc_type, exc_value, traceback)
+            finally:
+                torch.cuda.nvtx.range_pop()
+
+    for home in _RECORD_FUNCTION_HOMES:
+        module = importlib.import_module(home)
+        _original_record_functions[home] = module.record_function
+        module.record_function = marker_record_function
+
+
+def _restore_record_function() -> None:
+    import importlib
+
+    for home, original in _original_record_functions.items():
+        importlib.import_module(home).record_function = original
+    _original_record_functions.clear()
+
+
 def patch_fsdp2(enable_hpz: bool = False, compute_dtype_shards: Optional[bool] = None) -> None:
     """Create the two services and route torch's fully_shard collectives through them
     (fsdp2.py:1105-1138). Modules sharded afterwards need ``patch_lazy_init(module)`` each.
@@ -709,6 +752,8 @@ def patch_fsdp2(enable_hpz: bool = False, compute_dtype_shards: Optional[bool] =
         module.foreach_all_gather = foreach_all_gather
         module.foreach_all_gather_copy_out = foreach_all_gather_copy_out
         module.foreach_reduce = foreach_reduce
+    if os.environ.get("ODC_TRACE", "0") == "1":
+        _forward_record_function_to_markers()
     reduction_service = ReductionService()
     gather_service = GatherService()
 
@@ -726,6 +771,7 @@ def unpatch_fsdp2() -> None:
     if hasattr(comm_context, "_odc_original_lazy_init"):
         comm_context.lazy_init = comm_context._odc_original_lazy_init
         del comm_context._odc_original_lazy_init
+    _restore_record_function()
 
 
 def stop():

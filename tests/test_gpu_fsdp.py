@@ -249,3 +249,36 @@ def test_odc_all_gather_comm_object(make_world):
         assert_bit_equal(out, oracle.gather(shards), "async form after wait()")
     finally:
         fsdp2.unpatch_fsdp2()
+
+
+def test_record_function_ranges_become_marker_ranges_under_trace(monkeypatch):
+    """``ODC_TRACE=1``: ``patch_fsdp2`` installs a ``record_function`` that also opens a marker
+    range, in the three places the reference patches (fsdp2.py:1131-1133); the ranges still nest
+    and close, and ``unpatch_fsdp2`` puts torch's class back. Without the switch nothing changes."""
+    import torch.autograd.profiler
+    import torch.profiler
+    from torch.distributed.fsdp._fully_shard import _fsdp_param_group
+
+    from odc_amd.fsdp import fsdp2
+
+    original = torch.autograd.profiler.record_function
+    homes = (_fsdp_param_group, torch.profiler, torch.autograd.profiler)
+    fsdp2.patch_fsdp2()
+    assert all(h.record_function is original for h in homes)
+    fsdp2.unpatch_fsdp2()
+    monkeypatch.setenv("ODC_TRACE", "1")
+    fsdp2.patch_fsdp2()
+    try:
+        patched = _fsdp_param_group.record_function
+        assert patched is not original and issubclass(patched, original)
+        assert all(h.record_function is patched for h in homes)
+        pushed = []
+        monkeypatch.setattr(torch.cuda.nvtx, "range_push", lambda name: pushed.append(("push", name)))
+        monkeypatch.setattr(torch.cuda.nvtx, "range_pop", lambda: pushed.append(("pop",)))
+        with torch.profiler.record_function("FSDP::outer"):
+            with _fsdp_param_group.record_function("FSDP::inner"):
+                torch.ones(4, device="cuda").sum()
+        assert pushed == [("push", "FSDP::outer"), ("push", "FSDP::inner"), ("pop",), ("pop",)]
+    finally:
+        fsdp2.unpatch_fsdp2()
+    assert all(h.record_function is original for h in homes)

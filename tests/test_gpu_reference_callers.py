@@ -423,3 +423,41 @@ def test_example_reduce_scatter(make_world, lazy):
         )
         assert_bit_equal(reduction_service.accumulations[i], nccl_accumulations[i], f"accumulations[{i}]")
     assert reduction_service.stop() is None
+
+
+def test_the_reference_import_lines_work_unchanged(make_world):
+    """The import statements of the reference's callers, verbatim (examples/all_gather.py:10-11,
+    examples/reduce_scatter.py:9-10, examples/FSDP2/example.py:15-17, examples/llm_training's
+    ``import odc`` / ``from odc.fsdp import fsdp1``), give the objects of this package, and the
+    reference's known-answer gather (examples/all_gather.py:80-84,121-125: shard i of rank r holds
+    i + 2r) runs through them."""
+    import odc
+    from odc import init_nvshmem
+    from odc.fsdp import fsdp1 as ref_fsdp1
+    from odc.fsdp import fsdp2 as ref_fsdp2
+    from odc.primitives.gather import GatherService as RefGatherService
+    from odc.primitives.scatter_accumulate import ReductionService as RefReductionService
+    from odc.primitives.utils import SymmBufferRegistry as RefRegistry
+    from odc.primitives.utils import finalize_distributed, get_local_world_size, init_nvshmem as init_from_utils
+
+    import odc_amd
+    import odc_amd.primitives.utils as amd_utils
+
+    assert RefGatherService is GatherService and RefReductionService is ReductionService
+    assert RefRegistry is SymmBufferRegistry and ref_fsdp1 is fsdp1 and ref_fsdp2 is fsdp2
+    assert init_nvshmem is init_from_utils is odc_amd.init_nvshmem and odc.init_nvshmem is init_nvshmem
+    assert finalize_distributed is amd_utils.finalize_distributed
+    assert get_local_world_size is amd_utils.get_local_world_size
+    assert odc.ReductionService is ReductionService and odc.primitives.utils is amd_utils
+
+    group = make_world(W, 4 << 20)
+    registry = RefRegistry.get_instance()
+    gather = RefGatherService()
+    n = 4096
+    for r in range(W):
+        with odc.virtual_rank(r):
+            registry.update_symm_buffer(0, torch.full((n,), 0 + 2 * r, dtype=torch.int64, device="cuda"))
+    out = torch.empty(W * n, dtype=torch.int64, device="cuda")
+    gather.gather_into_tensor(out, registry.get_symm_buffer(0), group)
+    for r in range(W):
+        assert (out[r * n : (r + 1) * n] == 2 * r).all()

@@ -409,3 +409,25 @@ def test_under_the_sanitizer_run_the_sanitized_library_is_the_one_loaded():
     maps = open("/proc/self/maps").read()
     assert os.environ["ODC_HIP_LIBRARY"] in maps and "libasan" in maps
     assert str(_native.CSRC_DIR / "libodc_hip.so") not in maps
+
+
+def test_the_reference_module_paths_resolve_to_this_package():
+    """``odc`` is an alias package without logic: the module paths the reference's callers import
+    (examples/all_gather.py:10-11, examples/reduce_scatter.py:9-10, examples/FSDP2/example.py:15-17)
+    are the odc_amd modules themselves."""
+    import importlib
+
+    import odc
+    import odc_amd
+
+    for name in ("primitives", "primitives.gather", "primitives.scatter_accumulate", "primitives.utils",
+                 "primitives.tensor_ipc", "fsdp", "fsdp.fsdp1", "fsdp.fsdp2"):
+        assert importlib.import_module(f"odc.{name}") is importlib.import_module(f"odc_amd.{name}"), name
+    from odc.fsdp import fsdp2
+    from odc.primitives.gather import GatherService
+    from odc.primitives.utils import SymmBufferRegistry, init_nvshmem
+
+    assert GatherService is odc_amd.GatherService and SymmBufferRegistry is odc_amd.SymmBufferRegistry
+    assert init_nvshmem is odc_amd.init_nvshmem is odc.init_nvshmem and fsdp2.patch_fsdp2
+    text = (ROOT / "odc" / "__init__.py").read_text()
+    assert "def " not in text and "class " not in text, "the alias package holds no logic"
