@@ -177,7 +177,9 @@ int odc_convert(odc_arena* arena, const odc_convert_item* items, uint32_t n_item
  * widening, rounded to acc_dtype with round-to-nearest-even when acc_dtype is 16 bit. This is
  * acc[start:start+size].add_(buf[:size]) over all sub-buffers (scatter_accumulate.py:381-391)
  * fused with the staging copies (scatter_accumulate.py:649-669); the zero tail is the F.pad of
- * odc/fsdp/fsdp1.py:25-38.
+ * odc/fsdp/fsdp1.py:25-38. The items of one call must not overlap each other in the accumulations
+ * (they are worked on concurrently, in an order of the library's choosing: items of less than one
+ * tile per rank go last).
  * ---------------------------------------------------------------------------------------- */
 typedef struct odc_accum_item {
   const void* grad;      /* device pointer to the full gradient, grad_dtype */
@@ -241,7 +243,7 @@ int odc_abi_version(void);
  *    "publish_blocks_per_cu": persistent workgroups per CU walking the tiles with a grid-stride
  *    loop; 0 = one workgroup per tile, dealt out by the hardware dispatcher. accum_blocks_per_cu
  *    defaults to -1: one per tile, except 1 persistent per CU when the launch's segments average
- *    fewer than "accum_persistent_below_tiles" (128) tiles.
+ *    fewer than "accum_persistent_below_tiles" tiles (default 0: never).
  *  - "gather_resident_cap", "cast_resident_cap", "accum_resident_cap", "store_resident_cap",
  *    "publish_resident_cap": for one-workgroup-per-tile launches, the most workgroups resident per
  *    CU (enforced by claiming unused LDS; 0 = no cap, no claim; all default to 0).

@@ -20,6 +20,7 @@
 #include <mutex>
 #include <new>
 #include <string>
+#include <vector>
 
 #include "odc_hip.h"
 #include "odc_launch.h"
@@ -60,7 +61,7 @@ struct Options {
   int64_t accum_resident_cap = 0;
   int64_t accum_blocks_per_cu = -1;  // -1: by segment length (see scatter_launch)
   int64_t accum_short_segment_tiles = 256;   // segments averaging fewer tiles: rank-outermost tile order
-  int64_t accum_persistent_below_tiles = 128;  // segments averaging fewer tiles: persistent launch shape
+  int64_t accum_persistent_below_tiles = 0;  // segments averaging fewer tiles: persistent launch shape (0: never)
   int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
   int64_t store_resident_cap = 0;  // 512-thread workgroups, like the gathers
   int64_t clear_blocks_per_cu = 0;
@@ -453,13 +454,17 @@ int dtype_bytes(int dt) {
 }
 
 // odc_tiles::fill_tile_table with its failure turned into an error message.
+// `order`, when given, maps positions of the launch order to the caller's item indices (for the
+// message only: units and take already work on positions).
 template <class Units, class Take>
 int fill_launch(TileTable& tt, uint32_t world, uint32_t n_items, uint32_t* next, uint64_t tile_units,
-                Units units, Take take) {
+                Units units, Take take, const uint32_t* order = nullptr) {
   const int n = fill_tile_table(tt, world, n_items, next, tile_units, units, take);
-  if (n < 0)
-    return fail(ODC_ERR_INVALID, "item %d: %llu units per rank is too large for one launch", -1 - n,
-                (unsigned long long)units((uint32_t)(-1 - n)));
+  if (n < 0) {
+    const uint32_t at = (uint32_t)(-1 - n);
+    return fail(ODC_ERR_INVALID, "item %u: %llu units per rank is too large for one launch", order ? order[at] : at,
+                (unsigned long long)units(at));
+  }
   return n;
 }
 
@@ -644,7 +649,9 @@ int odc_clear(odc_arena* a, const odc_span* spans, uint32_t n_spans, void* strea
     ClearLaunch L;
     L.base = a->origin;
     L.rank_stride = a->rank_stride;
-    L.tt.order = kRanksInterleaved;  // a write-only stream runs fastest with the ranks interleaved
+    // a write-only stream runs fastest with the ranks interleaved (measured after an accumulate, as
+    // in a step: 117 us at W=64 against 123 item-major and 127 rank-outermost; level at W=128)
+    L.tt.order = kRanksInterleaved;
     L.tt.first_rank = 0;
     const int n = fill_launch(
         L.tt, a->world, n_spans, &next, kTileBytes, [&](uint32_t i) { return spans[i].nbytes; },
@@ -694,6 +701,26 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
       return fail(ODC_ERR_INVALID, "item %u: grad pointer is not aligned to the gradient dtype", i);
   }
   const Options opt = options_snapshot();
+  // Launch order of the items: those of less than one tile per rank go last. A tiny segment
+  // between two long ones (a norm vector's 64-element slice between two projection matrices)
+  // slows the read-modify-write stream around it out of all proportion to its size; at the end
+  // of the list it costs nothing (measured on the 8B layer, 9 items: -0.6 % of the launch time at
+  // W=64, -1.2 % at W=32, -5 % at W=128, nothing at W=8, where there are 16 such tiles instead of
+  // 128 or more; the gathers, the clear and the store form do not care). Items of one call are
+  // disjoint, so their order never changes the result.
+  uint32_t order_inline[256];
+  std::vector<uint32_t> order_heap;
+  uint32_t* order = order_inline;
+  if (n_items > 256) {
+    order_heap.resize(n_items);
+    order = order_heap.data();
+  }
+  {
+    uint32_t k = 0;
+    for (int small = 0; small < 2; ++small)
+      for (uint32_t i = 0; i < n_items; ++i)
+        if ((items[i].shard_elems < kTileElems) == (small != 0)) order[k++] = i;
+  }
   uint32_t next = 0;
   while (next < n_items) {
     AccumLaunch L;
@@ -702,11 +729,12 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     L.tt.order = (uint32_t)opt.rank_major;
     L.tt.first_rank = 0;
     const int n = fill_launch(
-        L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[i].shard_elems; },
+        L.tt, a->world, n_items, &next, kTileElems, [&](uint32_t i) { return items[order[i]].shard_elems; },
         [&](uint32_t slot, uint32_t i) {
-          L.item[slot] = {static_cast<const uint8_t*>(items[i].grad), items[i].grad_elems, items[i].acc_offset,
-                          items[i].shard_elems};
-        });
+          const odc_accum_item& it = items[order[i]];
+          L.item[slot] = {static_cast<const uint8_t*>(it.grad), it.grad_elems, it.acc_offset, it.shard_elems};
+        },
+        order);
     if (n < 0) return n;
     if (n == 0) continue;
     // Tile order. Item-major (a rank's segment, then the next rank's, item by item) walks the
@@ -721,16 +749,15 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
       L.tt.order = L.tt.n_tiles < (uint64_t)opt.accum_short_segment_tiles * segments ? kRankOutermost : kItemMajor;
     else
       L.tt.order = (uint32_t)opt.accum_tile_order;
-    // Launch shape. With tile-aligned rank regions and buffers, one workgroup per tile streams
-    // fastest down to segments of a few hundred tiles (measured: +1.0..2.3 % over the persistent
-    // shape at W=4..32). The persistent shape, one workgroup per CU, wins on shorter segments
-    // (+1.6 % at W=64, 92 tiles per segment; level at W=128), but only while every rank's chunk of
-    // the gradient and of the accumulation starts on a 128 B line: with nothing else resident to
-    // cover for it, a workgroup whose wavefronts straddle lines, or that meets heads, tails and
-    // padding, falls behind (measured: -7 % on 16 B aligned uneven shards). So: ragged launches
-    // and all but the shortest segments run one workgroup per tile.
-    // (Measured for 16-bit gradients into fp32 accumulations; fp32 gradients, 12 B per element,
-    // run 2 % faster one workgroup per tile.)
+    // Launch shape: one workgroup per tile. A persistent shape (one workgroup per CU,
+    // "accum_blocks_per_cu" = 1, or automatically below "accum_persistent_below_tiles" tiles per
+    // segment) used to win on very short segments (+1.6 % at W=64) only because it suffered less
+    // from tiny segments in the middle of the tile order; with those moved to the end the two
+    // shapes are level at W=64 and W=128 and one workgroup per tile is ahead everywhere else
+    // (W=16: +1.5 %, W=32: +0.9 %), and it is the shape that co-runs with compute kernels
+    // without starving them. A persistent grid is never used for ragged launches (a lone
+    // workgroup that straddles lines or meets heads, tails and padding falls behind: -7 % on
+    // 16 B aligned uneven shards) nor for other dtype pairs than 16-bit gradients into fp32.
     bool ragged = !(gb == 2 && ab == 4);
     for (uint32_t k = 0; k < L.tt.n_items; ++k)
       ragged |= (L.item[k].acc_off & 127u) != 0 || ((L.item[k].seg_elems * ab) & 127u) != 0 ||

@@ -483,3 +483,34 @@ def test_launch_stream_policies(make_world, monkeypatch, policy):
     monkeypatch.setenv("ODC_COMM_STREAM", "sideways")
     with pytest.raises(ValueError):
         gather.gather_into_tensor(out, src, group)
+
+
+@pytest.mark.parametrize("store", [False, True])
+def test_long_lists_mixing_tiny_and_large_items(make_world, store):
+    """300 keys in ONE call, every third of less than one tile per rank (those are launched after
+    the others, and a list this long takes the heap-allocated launch order and five launches):
+    every key gets exactly its own gradient, twice, in the read-modify-write form and after a lazy
+    clear in the store form."""
+    W = 4
+    group = make_world(W, 64 << 20)
+    _, _, registry = services()
+    from odc_amd import ReductionService
+
+    reduction = ReductionService(accumulation_dtype=torch.float32, lazy_clear=store)
+    g = torch.Generator().manual_seed(31)
+    sizes = [(7 + i if i % 3 == 0 else 4096 + 17 * i) for i in range(300)]
+    keys = [f"k{i}" for i in range(len(sizes))]
+    grads = [(torch.randn(W * s, generator=g) * 1e-3).bfloat16() for s in sizes]
+    dev = [t.cuda() for t in grads]
+    for k, s in zip(keys, sizes):
+        reduction.register(k, (s,), torch.bfloat16, torch.float32, group)
+    reduction.clear_accumulations()
+    reduction.scatter_accumulate_multi(keys, dev, group)
+    reduction.scatter_accumulate_multi(keys, dev, group)
+    reduction.sync(group)
+    for k, s, t in zip(keys, sizes, grads):
+        want = [torch.zeros(s) for _ in range(W)]
+        oracle.scatter_accumulate(want, t)
+        oracle.scatter_accumulate(want, t)
+        for r, acc in enumerate(reduction.get_peer_accumulations(k)):
+            assert_bit_equal(acc, want[r], f"key {k} rank {r}")

@@ -94,23 +94,30 @@ def test_long_item_lists_are_split_over_launches(arena, n_items):
 def test_accumulate_launch_shapes(arena):
     W = 8
     a = arena(W)
-    # line-aligned whole shards in SHORT segments (under 128 tiles each on average): the persistent
-    # shape, one workgroup per CU
+    # line-aligned whole shards in short segments: one workgroup per tile by default; the persistent
+    # shape, one workgroup per CU, only when asked for through the threshold
     shard = 1 << 18
     items = (_native.AccumItem * 2)(
         _native.AccumItem(OUTSIDE, W * shard, 0, shard), _native.AccumItem(OUTSIDE + (1 << 30), W * shard, 4 * shard, shard)
     )
     _native.check(a.lib.odc_scatter_accumulate(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
     launches, tiles, workgroups = a.counters()
-    assert (launches, tiles, workgroups) == (1, 2 * W * shard // TILE_ELEMS, N_CU)
-    # the same as a store, or with a gradient that ends early (padding): one workgroup per tile
+    assert (launches, tiles, workgroups) == (1, 2 * W * shard // TILE_ELEMS, 2 * W * shard // TILE_ELEMS)
     _native.set_option("dry_run_reset", 0)
-    _native.check(a.lib.odc_scatter_store(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
-    assert a.counters() == (1, tiles, tiles)
-    _native.set_option("dry_run_reset", 0)
-    items[1].grad_elems -= 5
-    _native.check(a.lib.odc_scatter_accumulate(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
-    assert a.counters() == (1, tiles, tiles)
+    _native.set_option("accum_persistent_below_tiles", 128)  # segments of 64 tiles are below it
+    try:
+        _native.check(a.lib.odc_scatter_accumulate(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+        assert a.counters() == (1, tiles, N_CU)
+        # the same as a store, or with a gradient that ends early (padding): one workgroup per tile
+        _native.set_option("dry_run_reset", 0)
+        _native.check(a.lib.odc_scatter_store(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+        assert a.counters() == (1, tiles, tiles)
+        _native.set_option("dry_run_reset", 0)
+        items[1].grad_elems -= 5
+        _native.check(a.lib.odc_scatter_accumulate(a.handle, items, 2, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+        assert a.counters() == (1, tiles, tiles)
+    finally:
+        _native.set_option("accum_persistent_below_tiles", 0)
     # long segments (128 tiles and more): one workgroup per tile, unless the knob says otherwise
     _native.set_option("dry_run_reset", 0)
     shard = 1 << 20
@@ -268,3 +275,29 @@ def test_arena_size_plus_alignment_slack_cannot_wrap():
         _native.check(lib.odc_arena_destroy(handle))
     finally:
         _native.set_option("rank_stride_align", 16384)
+
+
+@pytest.mark.parametrize("n_items", [5, 256, 257, 700])
+def test_accumulate_item_lists_with_tiny_items_keep_every_item(arena, n_items):
+    """Items of less than one tile per rank are launched after the others (also through the
+    heap-allocated order of lists longer than 256): launches and tiles still add up, and an item
+    that is too large is still reported under the caller's index."""
+    W = 4
+    a = arena(W, 1 << 46)
+    sizes = [(100 if i % 3 == 0 else 0 if i % 7 == 0 else 5000 + i) for i in range(n_items)]
+    items = (_native.AccumItem * n_items)()
+    off = 0
+    for it, sz in zip(items, sizes):
+        it.grad, it.grad_elems, it.acc_offset, it.shard_elems = OUTSIDE, W * sz, off, sz
+        off += -(-4 * sz // 256) * 256
+    _native.check(a.lib.odc_scatter_accumulate(a.handle, items, n_items, _native.DTYPE_BF16, _native.DTYPE_F32, None))
+    nonempty = [s for s in sizes if s]
+    launches, tiles, _ = a.counters()
+    assert launches == math.ceil(len(nonempty) / _native.MAX_ITEMS_PER_LAUNCH)
+    assert tiles == W * sum(math.ceil(s / TILE_ELEMS) for s in nonempty)
+    bad = n_items - 2  # position in the caller's list; in launch order it sits elsewhere
+    items[bad].shard_elems = (1 << 31) * TILE_ELEMS // W  # 2^31 tiles in all: one too many for a launch
+    items[bad].grad_elems, items[bad].acc_offset = 0, 0
+    status = a.lib.odc_scatter_accumulate(a.handle, items, n_items, _native.DTYPE_BF16, _native.DTYPE_F32, None)
+    message = a.lib.odc_last_error().decode()
+    assert status == _native.ODC_ERR_INVALID and f"item {bad}:" in message and "too large for one launch" in message
