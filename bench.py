@@ -82,10 +82,12 @@ def parse_args():
                          "timed scatter-accumulate is the 10N read-modify-write")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one torch copy of 1 GiB (counter calibration under rocprofv3)")
-    ap.add_argument("--probe", choices=["alignment", "overlap"],
-                    help="instead of the benchmark, print one of two measurement tables: alignment (what a buffer "
+    ap.add_argument("--probe", choices=["alignment", "overlap", "tiny-items"],
+                    help="instead of the benchmark, print one of three measurement tables: alignment (what a buffer "
                          "shifted off the 16 KiB tile grid costs the scatter-accumulate and the gather), overlap (how "
-                         "much of a gather / scatter-accumulate hides behind a co-running GEMM, by launch shape)")
+                         "much of a gather / scatter-accumulate hides behind a co-running GEMM, by launch shape), "
+                         "tiny-items (what items of less than one tile per rank cost the scatter-accumulate by their "
+                         "place in the launch order; run it with --world-size 64)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="libodc_hip launch knob, e.g. accum_blocks_per_cu=4")
     return ap.parse_args()
@@ -575,6 +577,65 @@ def probe_alignment(args, repeats=9, launches=20):
     odc.finalize_distributed()
 
 
+def probe_tiny_items(args, launches=40):
+    """`--probe tiny-items`: the 9-parameter layer's scatter-accumulate, launched back to back, with
+    its two norm items (64 elements per rank at W=64: less than one tile) where the caller lists
+    them (between the projection matrices), launched last (the library's default), and left out;
+    one workgroup per tile and one persistent workgroup per CU; rank-outermost and item-major."""
+    import torch
+
+    import odc_amd as odc
+    from odc_amd import _native
+    from odc_amd.workloads import llama3_8b_layer_shapes, numel
+
+    W = args.world_size
+    torch.cuda.set_device(0)
+    shapes = llama3_8b_layer_shapes()
+    numels = {name: numel(s) for name, s in shapes}
+    group = odc.init_nvshmem(world_size=W, symmetric_size=sum(v // W * 4 + 32768 for v in numels.values()) + (8 << 20))
+    reduction = odc.ReductionService(accumulation_dtype=torch.float32)
+    grads = {name: torch.empty(v, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3) for name, v in numels.items()}
+    for name, v in numels.items():
+        reduction.register(name, (v // W,), torch.bfloat16, torch.float32, group)
+    lists = {"all 9 items": [name for name, _ in shapes],
+             "without the norm items": [name for name, s in shapes if len(s) > 1]}
+
+    def timed(keys):
+        g = [grads[k] for k in keys]
+        for _ in range(5):
+            reduction.scatter_accumulate_multi(keys, g, group)
+        torch.cuda.synchronize()
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+        events[0].record()
+        for i in range(launches):
+            reduction.scatter_accumulate_multi(keys, g, group)
+            events[i + 1].record()
+        torch.cuda.synchronize()
+        return statistics.fmean(a.elapsed_time(b) for a, b in zip(events, events[1:])) * 1e3
+
+    print(f"scatter-accumulate of the Llama-3-8B layer, W={W}, microseconds per launch (mean of {launches} back to back)")
+    print(f"{'items, launch order of the tiny ones':44s} {'tile order':16s} {'per tile':>9s} {'persistent':>11s}")
+    try:
+        for label, keys in lists.items():
+            for last in ((0, 1) if len(keys) == 9 else (1,)):
+                for order, order_name in ((2, "rank-outermost"), (1, "item-major")):
+                    row = []
+                    for blocks_per_cu in (0, 1):
+                        _native.set_option("accum_small_items_last", last)
+                        _native.set_option("accum_tile_order", order)
+                        _native.set_option("accum_blocks_per_cu", blocks_per_cu)
+                        row.append(timed(keys))
+                    where = "" if len(keys) != 9 else (", tiny last" if last else ", as listed")
+                    print(f"{label + where:44s} {order_name:16s} {row[0]:9.1f} {row[1]:11.1f}", flush=True)
+    finally:
+        _native.set_option("accum_small_items_last", 1)
+        _native.set_option("accum_tile_order", 3)
+        _native.set_option("accum_blocks_per_cu", -1)
+    torch.cuda.synchronize()
+    odc.SymmBufferRegistry.get_instance().finalize()
+    odc.finalize_distributed()
+
+
 def probe_overlap(args, gemm=8192, launches=8, repeats=5):
     """`--probe overlap`: how much of a gather / scatter-accumulate hides behind compute on ONE
     GPU. The reference hops to a side stream so that its data movement overlaps the model's compute
@@ -675,7 +736,7 @@ def main():
               "second GPU. Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if args.probe:
-        return (probe_alignment if args.probe == "alignment" else probe_overlap)(args)
+        return {"alignment": probe_alignment, "overlap": probe_overlap, "tiny-items": probe_tiny_items}[args.probe](args)
     if args.workload == "model":
         return model_sweep(args)
 

@@ -252,6 +252,8 @@ int odc_abi_version(void);
  *    2 = rank outermost: all items' segments of rank 0, then of rank 1, ... accum_tile_order 3,
  *    its default, picks 2 when segments average fewer than "accum_short_segment_tiles" (256)
  *    tiles and 1 otherwise.
+ *  - "accum_small_items_last" (default 1): scatter-accumulate and scatter-store launch the items
+ *    of less than one tile per rank after the others; 0 keeps the caller's order.
  *  - "rank_stagger_bytes" (extra distance between rank regions), "rank_stride_align" (rank regions
  *    start on multiples of it, default 16384 = one tile) and "alloc_align" (allocations of at
  *    least this many bytes start on multiples of it, default 16384; smaller ones on 256): read

@@ -62,6 +62,7 @@ struct Options {
   int64_t accum_blocks_per_cu = -1;  // -1: by segment length (see scatter_launch)
   int64_t accum_short_segment_tiles = 256;   // segments averaging fewer tiles: rank-outermost tile order
   int64_t accum_persistent_below_tiles = 0;  // segments averaging fewer tiles: persistent launch shape (0: never)
+  int64_t accum_small_items_last = 1;  // scatter launches: items of less than one tile per rank go last
   int64_t store_blocks_per_cu = 0;  // the scatter-store (no read of the accumulation)
   int64_t store_resident_cap = 0;  // 512-thread workgroups, like the gathers
   int64_t clear_blocks_per_cu = 0;
@@ -82,6 +83,7 @@ int64_t* option_slot(const char* name) {
   if (!strcmp(name, "accum_blocks_per_cu")) return &g_opt.accum_blocks_per_cu;
   if (!strcmp(name, "accum_short_segment_tiles")) return &g_opt.accum_short_segment_tiles;
   if (!strcmp(name, "accum_persistent_below_tiles")) return &g_opt.accum_persistent_below_tiles;
+  if (!strcmp(name, "accum_small_items_last")) return &g_opt.accum_small_items_last;
   if (!strcmp(name, "clear_blocks_per_cu")) return &g_opt.clear_blocks_per_cu;
   if (!strcmp(name, "publish_blocks_per_cu")) return &g_opt.publish_blocks_per_cu;
   if (!strcmp(name, "rank_major")) return &g_opt.rank_major;
@@ -719,7 +721,7 @@ int scatter_launch(odc_arena* a, const odc_accum_item* items, uint32_t n_items, 
     uint32_t k = 0;
     for (int small = 0; small < 2; ++small)
       for (uint32_t i = 0; i < n_items; ++i)
-        if ((items[i].shard_elems < kTileElems) == (small != 0)) order[k++] = i;
+        if ((opt.accum_small_items_last != 0 && items[i].shard_elems < kTileElems) == (small != 0)) order[k++] = i;
   }
   uint32_t next = 0;
   while (next < n_items) {
