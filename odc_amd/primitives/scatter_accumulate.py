@@ -162,7 +162,7 @@ class ReductionService:
         """Launch the clear kernel over ``keys`` (caller holds the lock)."""
         keys = list(keys)
         self._owed_zero.difference_update(keys)
-        if self._capture_scope:
+        if self._capture_scope and torch.cuda.is_current_stream_capturing():
             self._capture_scope.difference_update(keys)
         if not keys:
             return
@@ -256,7 +256,7 @@ class ReductionService:
 
     def _settle(self, keys):
         """Write the zeros still owed to ``keys`` (before anything reads or adds into them)."""
-        if self._capture_scope:
+        if self._capture_scope and torch.cuda.is_current_stream_capturing():
             deferred = [k for k in keys if k in self._capture_scope]
             if deferred:
                 self._clear_keys(deferred)  # recorded into the graph, in order
