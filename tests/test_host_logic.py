@@ -431,3 +431,40 @@ def test_the_reference_module_paths_resolve_to_this_package():
     assert init_nvshmem is odc_amd.init_nvshmem is odc.init_nvshmem and fsdp2.patch_fsdp2
     text = (ROOT / "odc" / "__init__.py").read_text()
     assert "def " not in text and "class " not in text, "the alias package holds no logic"
+
+
+def test_stream_order_waits_only_when_a_key_changes_streams(monkeypatch):
+    """``StreamOrder`` (the per-key memory of the last writing stream) on the CPU, with the two
+    functions that touch the GPU replaced: launches that stay on one stream join nothing; a key
+    that moves to another stream joins exactly the stream it was last written on, once; a launch
+    over all keys collapses the table; keys never seen count as written on the first stream."""
+    joins = []
+    monkeypatch.setattr(utils, "stream_from_handle", lambda handle: ("stream", handle))
+    monkeypatch.setattr(utils, "join_streams", lambda current, previous: joins.append((current[1], previous)))
+    order = utils.StreamOrder()
+    A, B, C = 0x10, 0x20, 0x30
+    for _ in range(3):
+        order.before_launch(["a", "b"], A, total=3)
+    assert joins == [] and not order._last
+    order.before_launch(["a"], B, total=3)          # a: A -> B
+    assert joins == [(B, A)]
+    order.before_launch(["a"], B, total=3)          # stays: nothing
+    order.before_launch(["b"], A, total=3)          # b never left A
+    assert joins == [(B, A)]
+    order.before_launch(["a", "b"], C, total=3)     # a from B, b from A: two joins, in any order
+    assert sorted(joins[1:]) == [(C, A), (C, B)]
+    joins.clear()
+    order.before_launch(["c"], C, total=3)          # c counts as written on the first stream, A
+    assert joins == [(C, A)]
+    assert not order._last and order._base == C, "all three keys on C: the table collapses"
+    joins.clear()
+    order.before_launch(["a"], A, total=3)
+    order.before_launch(["a", "b", "c"], B, all_keys=True, total=3)   # e.g. a clear of everything
+    assert sorted(joins) == [(A, C), (B, A), (B, C)]
+    assert not order._last and order._base == B
+    joins.clear()
+    order.before_launch(["b"], B, total=3)
+    assert joins == []
+    order.forget()
+    order.before_launch(["a"], C, total=3)
+    assert joins == [] and order._base == C
