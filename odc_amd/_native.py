@@ -261,6 +261,11 @@ def load() -> ctypes.CDLL:
                         f"{LIB_PATH} is missing and could not be built ({e}): run "
                         "`python -c 'import __graft_entry__ as g; g.build()'` (needs hipcc)"
                     ) from None
+            # torch ships a HIP runtime of its own and must load it before this library pulls in
+            # the system's by name: two HIP runtimes in one process do not both see the device
+            # (a program that imported this package before torch found "no ROCm-capable device")
+            import torch  # noqa: F401
+
             lib = ctypes.CDLL(str(LIB_PATH))
             try:
                 _declare(lib)

@@ -271,3 +271,25 @@ def test_a_service_kept_across_arenas_does_not_reuse_stale_plans(make_world):
         registry.finalize()
         utils.finalize_distributed()
     del reduction
+
+
+def test_importing_the_package_before_torch_still_finds_the_gpu():
+    """A fresh interpreter that imports odc_amd (which loads libodc_hip.so) BEFORE torch must end
+    up with ONE HIP runtime, torch's: the arena is created and torch sees the same device."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    code = "\n".join([
+        f"import sys; sys.path.insert(0, {str(root)!r})",
+        "assert 'torch' not in sys.modules",
+        "import odc",
+        "import torch",
+        "g = odc.init_nvshmem(world_size=2, symmetric_size=1 << 20)",
+        "t = odc.SymmBufferRegistry.get_instance().allocate_symm_buffer('k', (16,), torch.float32)",
+        "t.fill_(3.0); torch.cuda.synchronize(); assert float(t.sum()) == 48.0",
+        "odc.SymmBufferRegistry.get_instance().finalize(); odc.finalize_distributed(); print('ok')",
+    ])
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0 and "ok" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-2000:]

@@ -179,3 +179,161 @@ def test_gather_on_another_stream_waits_for_the_conversion(make_world):
         torch.cuda.synchronize()
         want = torch.cat([s.bfloat16() for s in shards])
         assert_bit_equal(out, want, f"step {step}")
+
+
+@pytest.mark.parametrize("lazy", [False, True])
+@pytest.mark.parametrize("seed", range(4))
+def test_random_schedules_over_streams_match_the_sequential_oracle(make_world, seed, lazy):
+    """One host thread issues a random schedule of whole-key accumulates, multi-key accumulates,
+    slice accumulates, clears and publishes, every call on a randomly chosen one of four streams
+    (the default stream included). The caller's order is the only order there is, so after every
+    minibatch all accumulations must equal the sequential oracle bit for bit."""
+    import random
+
+    from odc_amd import ReductionService
+
+    rng = random.Random(1000 * seed + lazy)
+    Wl, n = 4, 300_000
+    group = make_world(Wl, 96 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=lazy)
+    gen = torch.Generator().manual_seed(seed)
+    keys = ["a", "b", "c", "d"]
+    slices = [(0, 100_000), (100_000, 4096), (110_000, 150_000)]  # of key "s": two gaps
+    total_s = 280_000
+    pool = [(torch.randn(Wl * n, generator=gen) * 1e-3).bfloat16() for _ in range(6)]
+    pool_dev = [g.cuda() for g in pool]
+    slice_pool = [[(torch.randn(Wl * m, generator=gen) * 1e-3).bfloat16() for _, m in slices] for _ in range(3)]
+    slice_dev = [[g.cuda() for g in gs] for gs in slice_pool]
+    streams = [torch.cuda.default_stream()] + [torch.cuda.Stream() for _ in range(3)]
+    for k in keys:
+        red.register(k, (n,), torch.bfloat16, torch.float32, group)
+    red.scatter_accumulate_slices("s", slice_dev[0], [o for o, _ in slices], [m for _, m in slices], group,
+                                  accumulation_numel=total_s)
+    torch.cuda.synchronize()
+    want = {k: [torch.zeros(n) for _ in range(Wl)] for k in keys}
+    want["s"] = [torch.zeros(total_s) for _ in range(Wl)]
+    for minibatch in range(3):
+        with torch.cuda.stream(rng.choice(streams)):
+            red.clear_accumulations()
+        for accs in want.values():
+            for a in accs:
+                a.zero_()
+        for _ in range(rng.randrange(6, 14)):
+            op = rng.choice(["one", "multi", "slices", "publish"])
+            with torch.cuda.stream(rng.choice(streams)):
+                if op == "one":
+                    k, g = rng.choice(keys), rng.randrange(len(pool))
+                    red.scatter_accumulate(k, pool_dev[g], group)
+                    oracle.scatter_accumulate(want[k], pool[g])
+                elif op == "multi":
+                    ks = rng.sample(keys, rng.randrange(2, 5))
+                    gs = [rng.randrange(len(pool)) for _ in ks]
+                    red.scatter_accumulate_multi(ks, [pool_dev[g] for g in gs], group)
+                    for k, g in zip(ks, gs):
+                        oracle.scatter_accumulate(want[k], pool[g])
+                elif op == "slices":
+                    g = rng.randrange(len(slice_pool))
+                    red.scatter_accumulate_slices("s", slice_dev[g], [o for o, _ in slices], [m for _, m in slices], group)
+                    for (o, m), t in zip(slices, slice_pool[g]):
+                        oracle.scatter_accumulate([w[o : o + m] for w in want["s"]], t)
+                else:
+                    k = rng.choice(keys)
+                    red.publish([k], divisor=2.0)  # rank 0 halves its accumulation in place (exact)
+                    want[k][0] /= 2.0
+        red.sync(group)
+        for k, accs in want.items():
+            # reading settles what a lazy clear still owes a key that the minibatch never touched
+            for r, acc in enumerate(red.get_peer_accumulations(k)):
+                assert_bit_equal(acc, accs[r], f"seed {seed} minibatch {minibatch} key {k} rank {r}")
+
+
+def _keep_busy(stream, milliseconds=60):
+    """Queue a kernel that occupies ``stream`` for a while, so that whatever is queued behind it
+    starts long after work issued later on other streams would, if nothing ordered them."""
+    a = torch.randn(4096, 4096, device="cuda")
+    with torch.cuda.stream(stream):
+        start = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(int(milliseconds * 12)):  # a 4096^3 fp32 GEMM takes well over 80 us here
+            a = a @ a.clamp(-1e-3, 1e-3)
+    return a
+
+
+@pytest.mark.parametrize("lazy", [False, True])
+def test_order_is_the_callers_even_when_the_earlier_stream_is_busy(make_world, lazy):
+    """Deterministic form of the ordering test: the stream of the EARLIER call is kept busy, so
+    without the service's ordering the later calls (a clear, a publish that halves, another
+    accumulate, on other streams) would run first and leave different values, not just a
+    different rounding."""
+    from odc_amd import ReductionService
+
+    Wl, n = 4, 200_000
+    group = make_world(Wl, 32 << 20)
+    red = ReductionService(accumulation_dtype=torch.float32, lazy_clear=lazy)
+    gen = torch.Generator().manual_seed(12)
+    g1, g2, g3 = ((torch.randn(Wl * n, generator=gen) * 1e-3).bfloat16() for _ in range(3))
+    d1, d2, d3 = g1.cuda(), g2.cuda(), g3.cuda()
+    red.register("k", (n,), torch.bfloat16, torch.float32, group)
+    s1, s2, s3 = (torch.cuda.Stream() for _ in range(3))
+    torch.cuda.synchronize()
+
+    # accumulate g1 behind a busy stream, then halve on another stream, then add g2 on a third
+    red.clear_accumulations()
+    busy = _keep_busy(s1)
+    with torch.cuda.stream(s1):
+        red.scatter_accumulate("k", d1, group)
+    with torch.cuda.stream(s2):
+        red.publish(["k"], divisor=2.0)
+    with torch.cuda.stream(s3):
+        red.scatter_accumulate("k", d2, group)
+    red.sync(group)
+    want = [torch.zeros(n) for _ in range(Wl)]
+    oracle.scatter_accumulate(want, g1)
+    want[0] /= 2.0  # the publishing rank is rank 0
+    oracle.scatter_accumulate(want, g2)
+    for r in range(Wl):
+        assert_bit_equal(red._registry_peers("k")[r], want[r], f"accumulate, publish, accumulate: rank {r}")
+
+    # accumulate g3 behind a busy stream, then a new minibatch (clear) and g1 on other streams
+    busy = _keep_busy(s2)
+    with torch.cuda.stream(s2):
+        red.scatter_accumulate("k", d3, group)
+    with torch.cuda.stream(s3):
+        red.clear_accumulations()
+    with torch.cuda.stream(s1):
+        red.scatter_accumulate("k", d1, group)
+    red.sync(group)
+    want = [torch.zeros(n) for _ in range(Wl)]
+    oracle.scatter_accumulate(want, g1)
+    for r in range(Wl):
+        assert_bit_equal(red.get_peer_accumulations("k")[r], want[r], f"accumulate, clear, accumulate: rank {r}")
+    del busy
+
+
+def test_gather_waits_for_a_conversion_on_a_busy_stream(make_world):
+    """The conversion is queued behind a busy stream; the gather issued afterwards on another
+    stream must still read the converted shards, not the copy made before."""
+    from odc_amd import GatherService, SymmBufferRegistry
+
+    Wl, n = 4, 100_003
+    group = make_world(Wl, 16 << 20)
+    registry = SymmBufferRegistry.get_instance()
+    gather = GatherService()
+    registry.allocate_symm_buffer("master", (n,), torch.float32)
+    registry.allocate_symm_buffer("compute", (n,), torch.bfloat16)
+    gen = torch.Generator().manual_seed(9)
+    s_convert, s_gather = torch.cuda.Stream(), torch.cuda.Stream()
+    out = torch.empty(Wl * n, dtype=torch.bfloat16, device="cuda")
+    for step in range(2):
+        shards = [torch.randn(n, generator=gen) * 0.02 for _ in range(Wl)]
+        for peer, shard in zip(registry.peer_tensors["master"], shards):
+            peer.copy_(shard)
+        torch.cuda.synchronize()
+        busy = _keep_busy(s_convert)
+        with torch.cuda.stream(s_convert):
+            gather.convert_symm_buffer("compute", "master")
+        with torch.cuda.stream(s_gather):
+            gather.gather_into_tensor(out, registry.get_symm_buffer("compute"), group)
+        torch.cuda.synchronize()
+        assert_bit_equal(out, torch.cat([s.bfloat16() for s in shards]), f"step {step}")
+        del busy
