@@ -311,8 +311,9 @@ def test_order_is_the_callers_even_when_the_earlier_stream_is_busy(make_world, l
 
 
 def test_gather_waits_for_a_conversion_on_a_busy_stream(make_world):
-    """The conversion is queued behind a busy stream; the gather issued afterwards on another
-    stream must still read the converted shards, not the copy made before."""
+    """The conversion is queued behind a busy stream; gathers issued afterwards on other streams
+    (several: streams that share a hardware queue with the conversion's are ordered by the queue
+    itself) must still read the converted shards, not the copy made before."""
     from odc_amd import GatherService, SymmBufferRegistry
 
     Wl, n = 4, 100_003
@@ -322,8 +323,9 @@ def test_gather_waits_for_a_conversion_on_a_busy_stream(make_world):
     registry.allocate_symm_buffer("master", (n,), torch.float32)
     registry.allocate_symm_buffer("compute", (n,), torch.bfloat16)
     gen = torch.Generator().manual_seed(9)
-    s_convert, s_gather = torch.cuda.Stream(), torch.cuda.Stream()
-    out = torch.empty(Wl * n, dtype=torch.bfloat16, device="cuda")
+    s_convert = torch.cuda.Stream()
+    s_gathers = [torch.cuda.Stream() for _ in range(5)]
+    outs = [torch.empty(Wl * n, dtype=torch.bfloat16, device="cuda") for _ in s_gathers]
     for step in range(2):
         shards = [torch.randn(n, generator=gen) * 0.02 for _ in range(Wl)]
         for peer, shard in zip(registry.peer_tensors["master"], shards):
@@ -332,8 +334,11 @@ def test_gather_waits_for_a_conversion_on_a_busy_stream(make_world):
         busy = _keep_busy(s_convert)
         with torch.cuda.stream(s_convert):
             gather.convert_symm_buffer("compute", "master")
-        with torch.cuda.stream(s_gather):
-            gather.gather_into_tensor(out, registry.get_symm_buffer("compute"), group)
+        for stream, out in zip(s_gathers, outs):
+            with torch.cuda.stream(stream):
+                gather.gather_into_tensor(out, registry.get_symm_buffer("compute"), group)
         torch.cuda.synchronize()
-        assert_bit_equal(out, torch.cat([s.bfloat16() for s in shards]), f"step {step}")
+        want = torch.cat([s.bfloat16() for s in shards])
+        for k, out in enumerate(outs):
+            assert_bit_equal(out, want, f"step {step}, gather stream {k}")
         del busy
